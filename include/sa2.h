@@ -1,0 +1,138 @@
+/*
+ * sa2 — sliding-window 2-simplicial attention for AMD MI355X (gfx950), C ABI.
+ *
+ * This header is the drop-in boundary of the library.  Each entry point replaces
+ * one device launch (or launch group) that the reference issues from
+ * simplicial_attention/triton_two_simplicial_attention.py; the file:line of the
+ * replaced call is given with every function.  No C++ or framework types cross
+ * this boundary: plain pointers, sizes, strides and an opaque hipStream_t.
+ *
+ * Conventions
+ *   - Every activation is (batch, seq, heads, dim_head) with an innermost stride
+ *     of one element; the three outer strides are passed in elements.  This is
+ *     the layout "[b, s, k, h]" of the reference kernels
+ *     (triton_two_simplicial_attention.py:60-66).
+ *   - lse and delta are contiguous fp32 (batch, heads, seq), the layout of the
+ *     reference's M and D buffers (triton_two_simplicial_attention.py:66,740,825).
+ *   - Keys/values carry kv_heads heads; query head h reads kv head h / (heads /
+ *     kv_heads), the "(h g)" order of triton_two_simplicial_attention.py:1033-1034.
+ *     Gradients of keys/values are written with kv_heads heads (already summed
+ *     over the group).
+ *   - Attended set of query i:  i-w1 < j <= i  and  i-w2 < k <= i
+ *     (triton_two_simplicial_attention.py:191-193).  Only causal = 1 is defined.
+ *   - seq_len is arbitrary: rows past the end are masked in-kernel, so the caller
+ *     does not need the zero padding of triton_two_simplicial_attention.py:1042-1046.
+ *   - All calls are asynchronous on the given stream, allocate nothing, keep no
+ *     device state and may be issued from any host thread.  Buffers are owned by
+ *     the caller.  The device is the caller's current HIP device.
+ *   - Return value: SA2_OK or an sa2_status; sa2_last_error() gives a
+ *     thread-local message for the last failure on the calling thread.
+ */
+#ifndef SA2_H
+#define SA2_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SA2_VERSION 100
+
+typedef enum sa2_status {
+    SA2_OK = 0,
+    SA2_ERR_NULL_POINTER = 1,   /* a required pointer is NULL */
+    SA2_ERR_BAD_SHAPE = 2,      /* non-positive size, heads % kv_heads != 0, window < 1 */
+    SA2_ERR_UNSUPPORTED = 3,    /* dim_head, dtype or causal flag the kernels do not cover */
+    SA2_ERR_ALIGNMENT = 4,      /* pointer or stride breaks the 16-byte row alignment */
+    SA2_ERR_LAUNCH = 5          /* hipGetLastError() after a launch was not hipSuccess */
+} sa2_status;
+
+typedef enum sa2_dtype { SA2_BF16 = 0 } sa2_dtype;
+
+/* Problem geometry shared by every entry point. */
+typedef struct sa2_problem {
+    int32_t batch;
+    int32_t seq_len;
+    int32_t heads;      /* query heads */
+    int32_t kv_heads;   /* key/value heads, divides heads */
+    int32_t dim_head;   /* 64 or 128 */
+    int32_t w1;         /* window of the first key/value set  (reference default 512) */
+    int32_t w2;         /* window of the second key/value set (reference default 32)  */
+    int32_t causal;     /* must be 1 */
+    float   scale;      /* softmax scale, dim_head^-0.5 in the reference (:735) */
+    int32_t dtype;      /* sa2_dtype of the activations */
+} sa2_problem;
+
+/* A (batch, seq, heads, dim_head) activation: base pointer and element strides. */
+typedef struct sa2_tensor {
+    void   *ptr;
+    int64_t stride_b;
+    int64_t stride_n;
+    int64_t stride_h;
+} sa2_tensor;
+
+/* Library version (SA2_VERSION of the build). */
+int sa2_version(void);
+
+/* Message of the last failing call on this thread ("" if none). */
+const char *sa2_last_error(void);
+
+/* 1 if the kernels cover this configuration, else 0.  Replaces the silent limits
+ * of the reference (HEAD_DIM fixed to 64, w2 <= 32:
+ * triton_two_simplicial_attention.py:51,291,508,586). */
+int sa2_supported(int32_t dim_head, int32_t w1, int32_t w2, int32_t dtype);
+
+/* Forward.  Replaces the launch of two_simplicial_attn_fwd_kernel
+ * (triton_two_simplicial_attention.py:749-798; kernel :58-228).
+ * Writes out (same layout as q) and lse[b,h,n] = log sum exp of the scaled logits. */
+int sa2_fwd(const sa2_problem *prob,
+            const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
+            const sa2_tensor *v1, const sa2_tensor *v2,
+            const sa2_tensor *out, float *lse, void *hip_stream);
+
+/* delta[b,h,n] = sum_d out * dout.  Replaces backward_preprocess_do_o_dot
+ * (triton_two_simplicial_attention.py:834-849; kernel :230-286). */
+int sa2_bwd_delta(const sa2_problem *prob, const sa2_tensor *out, const sa2_tensor *dout,
+                  float *delta, void *hip_stream);
+
+/* dQ.  Replaces the dQ half of two_simplicial_attn_bwd_kv2q_kernel
+ * (triton_two_simplicial_attention.py:939-1004; kernel :515-712, dq at :697-699,709). */
+int sa2_bwd_dq(const sa2_problem *prob,
+               const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
+               const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *dout,
+               const float *lse, const float *delta,
+               const sa2_tensor *dq, void *hip_stream);
+
+/* dK1, dV1 (first key/value set, window w1).  Replaces two_simplicial_attn_bwd_kv1_kernel
+ * (triton_two_simplicial_attention.py:868-934; kernel :298-503). */
+int sa2_bwd_dkv1(const sa2_problem *prob,
+                 const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
+                 const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *dout,
+                 const float *lse, const float *delta,
+                 const sa2_tensor *dk1, const sa2_tensor *dv1, void *hip_stream);
+
+/* dK2, dV2 (second key/value set, window w2).  Replaces the dK2/dV2 half of the two
+ * passes of two_simplicial_attn_bwd_kv2q_kernel
+ * (triton_two_simplicial_attention.py:938-1004; kernel :515-712, :680-683, :695, :702-707). */
+int sa2_bwd_dkv2(const sa2_problem *prob,
+                 const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
+                 const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *dout,
+                 const float *lse, const float *delta,
+                 const sa2_tensor *dk2, const sa2_tensor *dv2, void *hip_stream);
+
+/* Whole backward: delta, dQ, dK1/dV1, dK2/dV2 in stream order.  Replaces the body
+ * of SlidingTwoSimplicialAttention.backward (triton_two_simplicial_attention.py:808-1006).
+ * delta_ws is a caller-owned fp32 (batch, heads, seq) workspace.  Gradients are
+ * written in the activation dtype and need no prior zeroing. */
+int sa2_bwd(const sa2_problem *prob,
+            const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
+            const sa2_tensor *v1, const sa2_tensor *v2,
+            const sa2_tensor *out, const sa2_tensor *dout, const float *lse, float *delta_ws,
+            const sa2_tensor *dq, const sa2_tensor *dk1, const sa2_tensor *dk2,
+            const sa2_tensor *dv1, const sa2_tensor *dv2, void *hip_stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SA2_H */

@@ -1,0 +1,236 @@
+// C ABI of libsa2: argument validation and kernel launches (see include/sa2.h).
+#include "sa2.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+
+#include "sa2_bwd.hpp"
+#include "sa2_common.hpp"
+#include "sa2_fwd.hpp"
+
+namespace {
+
+thread_local char g_err[256] = "";
+
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+int check_problem(const sa2_problem *p) {
+    if (!p) return fail(SA2_ERR_NULL_POINTER, "problem is NULL");
+    if (p->batch < 1 || p->seq_len < 1 || p->heads < 1 || p->kv_heads < 1)
+        return fail(SA2_ERR_BAD_SHAPE, "batch=%d seq_len=%d heads=%d kv_heads=%d must all be >= 1", p->batch, p->seq_len,
+                    p->heads, p->kv_heads);
+    if (p->heads % p->kv_heads != 0)
+        return fail(SA2_ERR_BAD_SHAPE, "heads=%d is not a multiple of kv_heads=%d", p->heads, p->kv_heads);
+    if (p->w1 < 1 || p->w2 < 1) return fail(SA2_ERR_BAD_SHAPE, "windows w1=%d w2=%d must be >= 1", p->w1, p->w2);
+    if (p->causal != 1) return fail(SA2_ERR_UNSUPPORTED, "only causal=1 is defined for the sliding windows");
+    if (p->dtype != SA2_BF16) return fail(SA2_ERR_UNSUPPORTED, "dtype %d is not supported (bf16 only)", p->dtype);
+    if (p->dim_head != 64 && p->dim_head != 128)
+        return fail(SA2_ERR_UNSUPPORTED, "dim_head=%d is not supported (64 or 128)", p->dim_head);
+    if (!(p->scale > 0.f) || !std::isfinite(p->scale)) return fail(SA2_ERR_BAD_SHAPE, "scale must be positive and finite");
+    if ((int64_t)p->batch * p->heads * ((p->seq_len + 31) / 32) > 0x7fffffffll)
+        return fail(SA2_ERR_BAD_SHAPE, "problem too large for a 1-D grid");
+    return SA2_OK;
+}
+
+int check_tensor(const sa2_tensor *t, const char *name) {
+    if (!t || !t->ptr) return fail(SA2_ERR_NULL_POINTER, "tensor %s is NULL", name);
+    if ((reinterpret_cast<uintptr_t>(t->ptr) & 15) != 0 || (t->stride_b & 7) != 0 || (t->stride_n & 7) != 0 ||
+        (t->stride_h & 7) != 0)
+        return fail(SA2_ERR_ALIGNMENT, "tensor %s: base pointer must be 16-byte aligned and strides multiples of 8 elements",
+                    name);
+    return SA2_OK;
+}
+
+sa2::DevTensor dev(const sa2_tensor *t) {
+    sa2::DevTensor d;
+    d.ptr = static_cast<char *>(t->ptr);
+    d.sb = t->stride_b * 2;
+    d.sn = t->stride_n * 2;
+    d.sh = t->stride_h * 2;
+    return d;
+}
+
+sa2::KParams base_params(const sa2_problem *p) {
+    sa2::KParams k{};
+    k.B = p->batch;
+    k.N = p->seq_len;
+    k.H = p->heads;
+    k.HK = p->kv_heads;
+    k.G = p->heads / p->kv_heads;
+    k.w1 = p->w1;
+    k.w2 = p->w2;
+    k.scale = p->scale;
+    k.scale_log2e = p->scale * sa2::kLog2e;
+    return k;
+}
+
+int after_launch(const char *what) {
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return fail(SA2_ERR_LAUNCH, "%s launch failed: %s", what, hipGetErrorString(e));
+    return SA2_OK;
+}
+
+#define SA2_TRY(expr)                  \
+    do {                               \
+        int rc_ = (expr);              \
+        if (rc_ != SA2_OK) return rc_; \
+    } while (0)
+
+}  // namespace
+
+extern "C" {
+
+int sa2_version(void) { return SA2_VERSION; }
+
+const char *sa2_last_error(void) { return g_err; }
+
+int sa2_supported(int32_t dim_head, int32_t w1, int32_t w2, int32_t dtype) {
+    return (dim_head == 64 || dim_head == 128) && w1 >= 1 && w2 >= 1 && dtype == SA2_BF16;
+}
+
+int sa2_fwd(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
+            const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *out, float *lse, void *hip_stream) {
+    SA2_TRY(check_problem(prob));
+    SA2_TRY(check_tensor(q, "q"));
+    SA2_TRY(check_tensor(k1, "k1"));
+    SA2_TRY(check_tensor(k2, "k2"));
+    SA2_TRY(check_tensor(v1, "v1"));
+    SA2_TRY(check_tensor(v2, "v2"));
+    SA2_TRY(check_tensor(out, "out"));
+    if (!lse) return fail(SA2_ERR_NULL_POINTER, "lse is NULL");
+    sa2::KParams k = base_params(prob);
+    k.q = dev(q);
+    k.k1 = dev(k1);
+    k.k2 = dev(k2);
+    k.v1 = dev(v1);
+    k.v2 = dev(v2);
+    k.o = dev(out);
+    k.lse = lse;
+    hipStream_t s = static_cast<hipStream_t>(hip_stream);
+    int grid = prob->batch * prob->heads * ((prob->seq_len + 127) / 128);
+    if (prob->dim_head == 128)
+        hipLaunchKernelGGL(sa2::fwd_kernel<128>, dim3(grid), dim3(256), 0, s, k);
+    else
+        hipLaunchKernelGGL(sa2::fwd_kernel<64>, dim3(grid), dim3(256), 0, s, k);
+    return after_launch("forward");
+}
+
+int sa2_bwd_delta(const sa2_problem *prob, const sa2_tensor *out, const sa2_tensor *dout, float *delta,
+                  void *hip_stream) {
+    SA2_TRY(check_problem(prob));
+    SA2_TRY(check_tensor(out, "out"));
+    SA2_TRY(check_tensor(dout, "dout"));
+    if (!delta) return fail(SA2_ERR_NULL_POINTER, "delta is NULL");
+    sa2::KParams k = base_params(prob);
+    k.o = dev(out);
+    k.dout = dev(dout);
+    k.delta = delta;
+    hipStream_t s = static_cast<hipStream_t>(hip_stream);
+    int64_t rows = (int64_t)prob->batch * prob->heads * prob->seq_len;
+    int lanes_per_row = prob->dim_head / 8;
+    int rows_per_block = 256 / lanes_per_row;
+    int grid = (int)((rows + rows_per_block - 1) / rows_per_block);
+    if (prob->dim_head == 128)
+        hipLaunchKernelGGL(sa2::delta_kernel<128>, dim3(grid), dim3(256), 0, s, k);
+    else
+        hipLaunchKernelGGL(sa2::delta_kernel<64>, dim3(grid), dim3(256), 0, s, k);
+    return after_launch("delta");
+}
+
+static int bwd_common(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
+                      const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *dout, const float *lse,
+                      const float *delta, sa2::KParams *k) {
+    SA2_TRY(check_problem(prob));
+    SA2_TRY(check_tensor(q, "q"));
+    SA2_TRY(check_tensor(k1, "k1"));
+    SA2_TRY(check_tensor(k2, "k2"));
+    SA2_TRY(check_tensor(v1, "v1"));
+    SA2_TRY(check_tensor(v2, "v2"));
+    SA2_TRY(check_tensor(dout, "dout"));
+    if (!lse) return fail(SA2_ERR_NULL_POINTER, "lse is NULL");
+    if (!delta) return fail(SA2_ERR_NULL_POINTER, "delta is NULL");
+    *k = base_params(prob);
+    k->q = dev(q);
+    k->k1 = dev(k1);
+    k->k2 = dev(k2);
+    k->v1 = dev(v1);
+    k->v2 = dev(v2);
+    k->dout = dev(dout);
+    k->lse = const_cast<float *>(lse);
+    k->delta = const_cast<float *>(delta);
+    return SA2_OK;
+}
+
+int sa2_bwd_dq(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
+               const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *dout, const float *lse,
+               const float *delta, const sa2_tensor *dq, void *hip_stream) {
+    sa2::KParams k;
+    SA2_TRY(bwd_common(prob, q, k1, k2, v1, v2, dout, lse, delta, &k));
+    SA2_TRY(check_tensor(dq, "dq"));
+    k.dq = dev(dq);
+    hipStream_t s = static_cast<hipStream_t>(hip_stream);
+    int grid = prob->batch * prob->heads * ((prob->seq_len + 127) / 128);
+    if (prob->dim_head == 128)
+        hipLaunchKernelGGL(sa2::bwd_dq_kernel<128>, dim3(grid), dim3(256), 0, s, k);
+    else
+        hipLaunchKernelGGL(sa2::bwd_dq_kernel<64>, dim3(grid), dim3(256), 0, s, k);
+    return after_launch("dq");
+}
+
+int sa2_bwd_dkv1(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
+                 const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *dout, const float *lse,
+                 const float *delta, const sa2_tensor *dk1, const sa2_tensor *dv1, void *hip_stream) {
+    sa2::KParams k;
+    SA2_TRY(bwd_common(prob, q, k1, k2, v1, v2, dout, lse, delta, &k));
+    SA2_TRY(check_tensor(dk1, "dk1"));
+    SA2_TRY(check_tensor(dv1, "dv1"));
+    k.dk1 = dev(dk1);
+    k.dv1 = dev(dv1);
+    hipStream_t s = static_cast<hipStream_t>(hip_stream);
+    int grid = prob->batch * prob->kv_heads * ((prob->seq_len + 127) / 128);
+    if (prob->dim_head == 128)
+        hipLaunchKernelGGL(sa2::bwd_dkv1_kernel<128>, dim3(grid), dim3(256), 0, s, k);
+    else
+        hipLaunchKernelGGL(sa2::bwd_dkv1_kernel<64>, dim3(grid), dim3(256), 0, s, k);
+    return after_launch("dk1/dv1");
+}
+
+int sa2_bwd_dkv2(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
+                 const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *dout, const float *lse,
+                 const float *delta, const sa2_tensor *dk2, const sa2_tensor *dv2, void *hip_stream) {
+    sa2::KParams k;
+    SA2_TRY(bwd_common(prob, q, k1, k2, v1, v2, dout, lse, delta, &k));
+    SA2_TRY(check_tensor(dk2, "dk2"));
+    SA2_TRY(check_tensor(dv2, "dv2"));
+    k.dk2 = dev(dk2);
+    k.dv2 = dev(dv2);
+    hipStream_t s = static_cast<hipStream_t>(hip_stream);
+    int grid = prob->batch * prob->kv_heads * ((prob->seq_len + 127) / 128);
+    if (prob->dim_head == 128)
+        hipLaunchKernelGGL(sa2::bwd_dkv2_kernel<128>, dim3(grid), dim3(256), 0, s, k);
+    else
+        hipLaunchKernelGGL(sa2::bwd_dkv2_kernel<64>, dim3(grid), dim3(256), 0, s, k);
+    return after_launch("dk2/dv2");
+}
+
+int sa2_bwd(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
+            const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *out, const sa2_tensor *dout,
+            const float *lse, float *delta_ws, const sa2_tensor *dq, const sa2_tensor *dk1, const sa2_tensor *dk2,
+            const sa2_tensor *dv1, const sa2_tensor *dv2, void *hip_stream) {
+    SA2_TRY(sa2_bwd_delta(prob, out, dout, delta_ws, hip_stream));
+    SA2_TRY(sa2_bwd_dq(prob, q, k1, k2, v1, v2, dout, lse, delta_ws, dq, hip_stream));
+    SA2_TRY(sa2_bwd_dkv1(prob, q, k1, k2, v1, v2, dout, lse, delta_ws, dk1, dv1, hip_stream));
+    SA2_TRY(sa2_bwd_dkv2(prob, q, k1, k2, v1, v2, dout, lse, delta_ws, dk2, dv2, hip_stream));
+    return SA2_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,99 @@
+// Shared device helpers for the gfx950 kernels of sliding-window 2-simplicial attention.
+//
+// Register-fragment conventions used by every kernel (wave64, v_mfma_f32_32x32x16_bf16):
+//   lane = 32*hf + c            (c = lane % 32, hf = lane / 32)
+//   A operand (32 x 16): lane holds row c,    k-slots 8*hf .. 8*hf+7
+//   B operand (16 x 32): lane holds column c, k-slots 8*hf .. 8*hf+7
+//   C/D       (32 x 32): register r of lane holds row 8*(r/4) + 4*hf + r%4, column c
+// A contraction is invariant under any permutation of its k index applied to both
+// operands, so the kernels are free to choose which data index sits in which k-slot.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace sa2 {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+
+// (batch, seq, heads, dim) activation with byte strides (innermost stride = 2 bytes).
+struct DevTensor {
+    char *ptr;
+    int64_t sb, sn, sh;
+};
+
+struct KParams {
+    DevTensor q, k1, k2, v1, v2, o, dout, dq, dk1, dk2, dv1, dv2;
+    float *lse;
+    float *delta;
+    int B, N, H, HK, G;   // G = H / HK query heads per key/value head
+    int w1, w2;
+    float scale;          // softmax scale
+    float scale_log2e;    // scale * log2(e)
+};
+
+__device__ __forceinline__ float as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
+__device__ __forceinline__ uint32_t as_u32(float f) { return __builtin_bit_cast(uint32_t, f); }
+
+__device__ __forceinline__ float bf16_lo(uint32_t w) { return as_f32(w << 16); }
+__device__ __forceinline__ float bf16_hi(uint32_t w) { return as_f32(w & 0xffff0000u); }
+
+// two floats -> packed bf16 pair, round to nearest even (v_cvt_pk_bf16_f32)
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    bf16x2 v = {(__bf16)lo, (__bf16)hi};
+    return __builtin_bit_cast(uint32_t, v);
+}
+
+__device__ __forceinline__ u32x4 ld_global16(const char *p) { return *reinterpret_cast<const u32x4 *>(p); }
+__device__ __forceinline__ void st_global16(char *p, u32x4 v) { *reinterpret_cast<u32x4 *>(p) = v; }
+__device__ __forceinline__ u32x4 ld_lds16(const char *p) { return *reinterpret_cast<const u32x4 *>(p); }
+
+__device__ __forceinline__ bf16x8 as_bf16x8(u32x4 v) { return __builtin_bit_cast(bf16x8, v); }
+
+// element-wise product of two packed bf16x8 fragments, rounded back to bf16
+__device__ __forceinline__ u32x4 mul_bf16x8(u32x4 a, u32x4 b) {
+    u32x4 r;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) r[w] = pack_bf16(bf16_lo(a[w]) * bf16_lo(b[w]), bf16_hi(a[w]) * bf16_hi(b[w]));
+    return r;
+}
+
+__device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(a), as_bf16x8(b), c, 0, 0, 0);
+}
+
+__device__ __forceinline__ f32x16 zero16() {
+    f32x16 z;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) z[r] = 0.f;
+    return z;
+}
+
+// value held by the lane with the same column in the other half of the wave
+__device__ __forceinline__ float other_half(float x) { return __shfl_xor(x, 32, 64); }
+
+__device__ __forceinline__ bool wave_any(bool pred) { return __builtin_amdgcn_ballot_w64(pred) != 0ull; }
+
+__device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// Storage position of row j (0..15 within an aligned group of 16) inside a
+// "k-slot ordered" transposed tile: rows 8a+4h+c (a,h in {0,1}, c in 0..3) sit at
+// 8h+4a+c, so that the 8 rows a C-layout lane of half h owns are contiguous.
+__device__ __forceinline__ int kslot_pos(int j) {
+    return (j & ~15) | ((j & 4) << 1) | ((j & 8) >> 1) | (j & 3);
+}
+
+// Grid index -> logical work item such that the eight XCDs (which receive
+// consecutive workgroup ids round-robin) each walk a contiguous range of items.
+__device__ __forceinline__ int xcd_contiguous(int wg, int total) {
+    return (total % 8 == 0) ? (wg % 8) * (total / 8) + wg / 8 : wg;
+}
+
+}  // namespace sa2

@@ -1,0 +1,93 @@
+"""Multi-head wrapper around a higher-order ``attend`` callable.
+
+Counterpart of simplicial_attention/simplicial_mha.py:28-150 of the reference: the
+same constructor arguments, the same parameter names and shapes (so a reference
+``state_dict`` loads unchanged) and the same channel order of the fused projection,
+``(head, set, d)`` for keys and values.
+"""
+from __future__ import annotations
+
+from functools import partial
+from typing import Callable
+
+from torch import nn
+
+from .naive import naive_two_simplicial_attend
+
+
+class HigherOrderAttention(nn.Module):
+    def __init__(
+        self,
+        dim,
+        causal=False,
+        dim_head=64,
+        dim_head_values=None,
+        heads=8,
+        key_value_heads=None,
+        number_key_value_sets=2,
+        qk_rmsnorm=True,
+        prenorm=False,
+        postnorm=False,
+        attend: Callable | None = None,
+        head_first_dim=True,
+    ):
+        super().__init__()
+        key_value_heads = heads if key_value_heads is None else key_value_heads
+        dim_head_values = dim_head if dim_head_values is None else dim_head_values
+        assert heads % key_value_heads == 0, 'heads must be a multiple of key_value_heads'
+
+        self.causal = causal
+        self.scale = dim_head ** -0.5
+        self.heads = heads
+        self.key_value_heads = key_value_heads
+        self.query_head_groups = heads // key_value_heads
+        self.kv_sets = number_key_value_sets
+        self.head_first_dim = head_first_dim
+        self.qk_rmsnorm = qk_rmsnorm
+
+        self.prenorm = nn.RMSNorm(dim) if prenorm else nn.Identity()
+        self.postnorm = nn.RMSNorm(dim) if postnorm else nn.Identity()
+        if qk_rmsnorm:
+            self.q_norm = nn.RMSNorm(dim_head)
+            self.k_norms = nn.ModuleList(nn.RMSNorm(dim_head) for _ in range(self.kv_sets))
+            self.v_norms = nn.ModuleList(nn.RMSNorm(dim_head) for _ in range(self.kv_sets))
+
+        self.split_dims = (heads * dim_head,
+                           self.kv_sets * key_value_heads * dim_head,
+                           self.kv_sets * key_value_heads * dim_head_values)
+        self.to_qkv = nn.Linear(dim, sum(self.split_dims), bias=False)
+        self.combine_heads = nn.Linear(heads * dim_head_values, dim, bias=False)
+
+        if attend is None:
+            if self.kv_sets != 2:
+                raise NotImplementedError('only two key/value sets have a built-in attend; pass attend=...')
+            attend = naive_two_simplicial_attend
+        if causal:
+            attend = partial(attend, causal=causal)
+        self.attend = attend
+
+    def _split(self, t, heads):
+        t = t.unflatten(-1, (heads, -1))                       # b n h d
+        return t.transpose(1, 2) if self.head_first_dim else t
+
+    def forward(self, tokens):
+        tokens = self.prenorm(tokens)
+        q, k, v = self.to_qkv(tokens).split(self.split_dims, dim=-1)
+        queries = self._split(q, self.heads)
+        keys = self._split(k, self.key_value_heads).chunk(self.kv_sets, dim=-1)
+        values = self._split(v, self.key_value_heads).chunk(self.kv_sets, dim=-1)
+        if self.qk_rmsnorm:
+            queries = self.q_norm(queries)
+            keys = tuple(norm(t) for norm, t in zip(self.k_norms, keys))
+            values = tuple(norm(t) for norm, t in zip(self.v_norms, values))
+        out = self.attend(queries, keys, values)
+        if self.head_first_dim:
+            out = out.transpose(1, 2)
+        out = self.combine_heads(out.flatten(-2))
+        return self.postnorm(out)
+
+
+class TwoSimplicialMHA(HigherOrderAttention):
+    def __init__(self, *args, **kwargs):
+        assert 'number_key_value_sets' not in kwargs
+        super().__init__(*args, number_key_value_sets=2, **kwargs)

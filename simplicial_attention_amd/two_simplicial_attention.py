@@ -1,0 +1,128 @@
+"""Sliding-window 2-simplicial attention on MI355X: autograd Function, functional
+wrapper and multi-head module.
+
+Same names, argument order, tensor layouts and defaults as
+simplicial_attention/triton_two_simplicial_attention.py of the reference
+(Function :718-1008, wrapper :1020-1056, module :1062-1081); the device work is done
+by hand-written gfx950 kernels reached through the C ABI of libsa2.so.
+"""
+from __future__ import annotations
+
+from functools import partial
+
+import torch
+from torch import Tensor
+from torch.autograd import Function
+
+from . import _native
+from .simplicial_mha import HigherOrderAttention
+
+
+def _unit_inner_stride(t: Tensor) -> Tensor:
+    """The kernels need a unit innermost stride, 16-byte aligned rows and base."""
+    ok = (t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all(s % 8 == 0 for s in t.stride()[:-1]))
+    return t if ok else t.contiguous()
+
+
+def _stream_handle(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+class SlidingTwoSimplicialAttention(Function):
+    """``apply(q, k1, k2, v1, v2, w1, w2, causal) -> out``; every tensor ``(b, n, h, d)``.
+
+    ``k1, k2, v1, v2`` may carry fewer heads than ``q`` (grouped queries, query head
+    ``h`` reads key/value head ``h // groups``); the reference's Function receives
+    them already repeated, which is the special case of one group per head.
+    Gradients come back in the order ``dq, dk1, dk2, dv1, dv2`` in the input dtype.
+    """
+
+    @staticmethod
+    def forward(ctx, q, k1, k2, v1, v2, w1, w2, causal):
+        tensors = (q, k1, k2, v1, v2)
+        assert all(t.is_cuda for t in tensors), 'sliding-window 2-simplicial attention runs on the GPU only'
+        if not causal:
+            raise NotImplementedError('only causal=True is defined for the sliding windows')
+        if any(t.dtype != torch.bfloat16 for t in tensors):
+            raise TypeError('the MI355X kernels take bfloat16 activations; cast inputs with .bfloat16()')
+        if q.dim() != 4:
+            raise ValueError('expected (batch, seq, heads, dim_head) tensors')
+        batch, seq_len, heads, dim = q.shape
+        kv_heads = k1.shape[2]
+        for t in (k1, k2, v1, v2):
+            if t.shape != (batch, seq_len, kv_heads, dim):
+                raise ValueError(f'key/value shape {tuple(t.shape)} does not match {(batch, seq_len, kv_heads, dim)}')
+        if heads % kv_heads != 0:
+            raise ValueError(f'query heads {heads} not divisible by key/value heads {kv_heads}')
+        w1, w2 = int(w1), int(w2)
+        if w1 < 1 or w2 < 1:
+            raise ValueError('window sizes must be at least 1')
+        lib = _native.load()
+        if not lib.sa2_supported(dim, w1, w2, _native.SA2_BF16):
+            raise NotImplementedError(f'dim_head={dim}, w1={w1}, w2={w2} is not covered by the kernels (dim_head 64 or 128)')
+
+        q, k1, k2, v1, v2 = (_unit_inner_stride(t) for t in tensors)
+        scale = dim ** -0.5
+        out = torch.empty((batch, seq_len, heads, dim), dtype=q.dtype, device=q.device)
+        lse = torch.empty((batch, heads, seq_len), dtype=torch.float32, device=q.device)
+        prob = _native.problem(batch, seq_len, heads, kv_heads, dim, w1, w2, True, scale)
+        with torch.cuda.device_of(q):
+            _native.check(lib.sa2_fwd(prob, *(_native.tensor_arg(t) for t in (q, k1, k2, v1, v2, out)),
+                                      lse.data_ptr(), _stream_handle(q.device)))
+        ctx.save_for_backward(q, k1, k2, v1, v2, out, lse)
+        ctx.problem = (batch, seq_len, heads, kv_heads, dim, w1, w2, scale)
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k1, k2, v1, v2, out, lse = ctx.saved_tensors
+        batch, seq_len, heads, kv_heads, dim, w1, w2, scale = ctx.problem
+        dout = _unit_inner_stride(dout)
+        lib = _native.load()
+        delta = torch.empty_like(lse)
+        dq = torch.empty_like(q)
+        dk1, dk2, dv1, dv2 = (torch.empty((batch, seq_len, kv_heads, dim), dtype=q.dtype, device=q.device) for _ in range(4))
+        prob = _native.problem(batch, seq_len, heads, kv_heads, dim, w1, w2, True, scale)
+        arg = _native.tensor_arg
+        with torch.cuda.device_of(q):
+            _native.check(lib.sa2_bwd(prob, arg(q), arg(k1), arg(k2), arg(v1), arg(v2), arg(out), arg(dout),
+                                      lse.data_ptr(), delta.data_ptr(),
+                                      arg(dq), arg(dk1), arg(dk2), arg(dv1), arg(dv2), _stream_handle(q.device)))
+        return dq, dk1, dk2, dv1, dv2, None, None, None
+
+
+_sliding_two_simplicial_attn = SlidingTwoSimplicialAttention.apply
+
+
+def sliding_two_simplicial_attn(
+    q: Tensor,                      # (b, n, hq, d)
+    keys: tuple[Tensor, Tensor],    # (b, n, h, d) * 2
+    values: tuple[Tensor, Tensor],  # (b, n, h, d) * 2
+    w1=512,
+    w2=32,
+    causal=True,
+    pad_to_multiple_of=64,
+):
+    """Functional entry point, signature of triton_two_simplicial_attention.py:1020-1056.
+
+    Grouped-query heads are resolved by index arithmetic inside the kernels and a
+    ragged sequence end is masked there, so nothing is repeated or padded here;
+    ``pad_to_multiple_of`` is accepted for compatibility and has no effect on the
+    result (zero rows appended after a causal sequence cannot influence it).
+    """
+    if len(keys) != 2 or len(values) != 2:
+        raise AssertionError('two key sets and two value sets are required')
+    q_heads, k_heads = q.shape[-2], keys[0].shape[-2]
+    assert q_heads % k_heads == 0, 'query heads must be a multiple of key/value heads'
+    (k1, k2), (v1, v2) = keys, values
+    return _sliding_two_simplicial_attn(q, k1, k2, v1, v2, w1, w2, causal)
+
+
+class SlidingWindowTwoSimplicialMHA(HigherOrderAttention):
+    """Multi-head module, constructor of triton_two_simplicial_attention.py:1062-1081."""
+
+    def __init__(self, *args, w1=512, w2=32, **kwargs):
+        assert 'number_key_value_sets' not in kwargs
+        assert 'head_first_dim' not in kwargs
+        attend = partial(sliding_two_simplicial_attn, w1=w1, w2=w2, causal=True)
+        super().__init__(*args, number_key_value_sets=2, head_first_dim=False, attend=attend, **kwargs)
