@@ -1,0 +1,193 @@
+#!/usr/bin/env python3
+"""Benchmark of sliding-window 2-simplicial attention on one MI355X.
+
+One step = one forward + backward of the raw kernel path over one batch of synthetic
+input (BASELINE config 3: B=4, H=8, N=8192, D=128, w1=512, w2=32, bf16; q, k1, k2, v1,
+v2 ~ N(0,1)/sqrt(D), dO ~ N(0,1)), called through the autograd Function with inputs
+resident in HBM.  Prints one JSON line.
+
+Algorithmic work (attended triples P per (batch, head), P = sum_i min(i+1,w1) min(i+1,w2)):
+    forward  4*D*P flop   (logit and value contraction)
+    backward 14*D*P flop  (S, dP, dV1, dV2, dK1, dK2, dQ)
+`value` uses 18*D*B*H*P over the fwd+bwd time.  Each kernel is also timed on its own
+through the C ABI with HIP events on the launch stream; the `roofline` object is for
+the kernel with the longest launch, priced with the contractions that kernel needs
+for its own outputs (fwd 2, dQ 3, dK1/dV1 4, dK2/dV2 4; 2*D flop each per triple).
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_BF16_TFLOPS = 2516.6   # MI355X dense bf16 MFMA peak
+PEAK_HBM_GBS = 8000.0
+
+WORKLOADS = {
+    # name: (B, H, HK, N, D, w1, w2)
+    'cfg3_raw_kernel_b4_h8_n8192_d128_w512_w32': (4, 8, 8, 8192, 128, 512, 32),
+    'cfg4_long_context_b1_h16_n32768_d128_w512_w32': (1, 16, 16, 32768, 128, 512, 32),
+    'cfg5_layer_b8_h8_kv4_n2048_d64_w512_w32': (8, 8, 4, 2048, 64, 512, 32),
+    'tiny_b1_h2_n512_d128_w512_w32': (1, 2, 2, 512, 128, 512, 32),
+}
+
+
+def attended_triples(n, w1, w2):
+    return sum(min(i + 1, w1) * min(i + 1, w2) for i in range(n))
+
+
+def cpu_baseline(N, D, w1, w2, slices):
+    """The banded fp32 CPU oracle (a port of the reference algorithm; the reference
+    has no CPU implementation of the windowed path) on `slices` complete (batch, head)
+    slices of the workload, forward + backward, timed once."""
+    import torch
+    from oracle import reference_attend as R
+    g = torch.Generator().manual_seed(2)
+    q, k1, k2, v1, v2 = [(torch.randn(1, N, slices, D, generator=g) * D ** -0.5).bfloat16().float() for _ in range(5)]
+    dout = torch.randn(1, N, slices, D, generator=g).bfloat16().float()
+    t0 = time.perf_counter()
+    R.windowed_banded_fwd_bwd(q, k1, k2, v1, v2, dout, w1, w2, chunk=64)
+    t = time.perf_counter() - t0
+    flops = 18 * D * slices * attended_triples(N, w1, w2)
+    return {
+        'value': round(flops / t / 1e12, 4), 'unit': 'TFLOP/s', 'cores': torch.get_num_threads(), 'kind': 'port',
+        'tokens_per_s': round(N * slices / t, 1),
+        'sample': f'{slices} of the workload\'s (batch, head) slices, all {N} rows each, D={D} w1={w1} w2={w2}, '
+                  f'fp32 banded oracle fwd+bwd, one run of {t:.1f} s; tokens_per_s counts rows of these slices; '
+                  f'host cpu_count={os.cpu_count()}',
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument('--gpus', type=int, default=1)
+    ap.add_argument('--steps', type=int, default=10)
+    ap.add_argument('--warmup', type=int, default=3)
+    ap.add_argument('--workload', default='cfg3_raw_kernel_b4_h8_n8192_d128_w512_w32', choices=sorted(WORKLOADS))
+    ap.add_argument('--cpu-slices', type=int, default=4, help='(batch, head) slices of the CPU baseline sample (0 = skip)')
+    ap.add_argument('--kernel-iters', type=int, default=5, help='launches per kernel for the per-kernel timing')
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print('bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path exists)', file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from simplicial_attention_amd import _native, sliding_two_simplicial_attn
+    if not torch.cuda.is_available():
+        print('bench.py: no GPU visible', file=sys.stderr)
+        sys.exit(1)
+    if not os.path.exists(_native.LIB_PATH):
+        import __graft_entry__
+        __graft_entry__.build()
+    lib = _native.load()
+
+    B, H, HK, N, D, w1, w2 = WORKLOADS[args.workload]
+    dev = torch.device('cuda:0')
+    g = torch.Generator(device='cpu').manual_seed(2)
+    mk = lambda h, s: (torch.randn(B, N, h, D, generator=g) * s).bfloat16().to(dev)
+    q = mk(H, D ** -0.5)
+    k1, k2, v1, v2 = (mk(HK, D ** -0.5) for _ in range(4))
+    dout = mk(H, 1.0)
+    ins = [t.requires_grad_(True) for t in (q, k1, k2, v1, v2)]
+
+    def fwd():
+        return sliding_two_simplicial_attn(ins[0], (ins[1], ins[2]), (ins[3], ins[4]), w1=w1, w2=w2, causal=True)
+
+    def step():
+        out = fwd()
+        return torch.autograd.grad(out, ins, dout)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    step_s = (time.perf_counter() - t0) / args.steps
+
+    # forward only (same API, no graph kept)
+    with torch.no_grad():
+        for _ in range(2):
+            fwd()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(max(3, args.steps)):
+            fwd()
+        torch.cuda.synchronize()
+        fwd_s = (time.perf_counter() - t0) / max(3, args.steps)
+
+    # ---- per-kernel timing through the C ABI, HIP events on the launch stream
+    P = attended_triples(N, w1, w2)
+    unit = 2 * D * B * H * P   # one contraction over all triples
+    stream = torch.cuda.current_stream()
+    sh = stream.cuda_stream
+    arg = _native.tensor_arg
+    prob = _native.problem(B, N, H, HK, D, w1, w2, True, D ** -0.5)
+    qd, k1d, k2d, v1d, v2d = (t.detach() for t in ins)
+    out = torch.empty_like(qd)
+    res = torch.empty_like(qd)
+    lse = torch.empty(B, H, N, dtype=torch.float32, device=dev)
+    delta = torch.empty_like(lse)
+    dq = torch.empty_like(qd)
+    dk1, dk2, dv1, dv2 = (torch.empty_like(k1d) for _ in range(4))
+    five = (arg(qd), arg(k1d), arg(k2d), arg(v1d), arg(v2d))
+    launches = {
+        'fwd': (2, lambda: lib.sa2_fwd(prob, *five, arg(out), arg(res), lse.data_ptr(), sh)),
+        'bwd_delta': (0, lambda: lib.sa2_bwd_delta(prob, arg(out), arg(res), arg(dout), delta.data_ptr(), sh)),
+        'bwd_dq': (3, lambda: lib.sa2_bwd_dq(prob, *five, arg(dout), lse.data_ptr(), delta.data_ptr(), arg(dq), sh)),
+        'bwd_dkv1': (4, lambda: lib.sa2_bwd_dkv1(prob, *five, arg(dout), lse.data_ptr(), delta.data_ptr(), arg(dk1), arg(dv1), sh)),
+        'bwd_dkv2': (4, lambda: lib.sa2_bwd_dkv2(prob, *five, arg(dout), lse.data_ptr(), delta.data_ptr(), arg(dk2), arg(dv2), sh)),
+    }
+    kernels = {}
+    for name, (ncontr, fn) in launches.items():
+        _native.check(fn())
+        torch.cuda.synchronize()
+        evs = []
+        for _ in range(args.kernel_iters):
+            a, b_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record(stream)
+            _native.check(fn())
+            b_.record(stream)
+            evs.append((a, b_))
+        torch.cuda.synchronize()
+        ms = statistics.mean(a.elapsed_time(b_) for a, b_ in evs)
+        kernels[name] = {'ms': round(ms, 4), 'contractions': ncontr,
+                         'tflops': round(ncontr * unit / (ms * 1e-3) / 1e12, 2) if ncontr else None}
+    hbm_bytes = {'fwd': 7 * B * N * H * D * 2 + 4 * B * H * N, 'bwd_delta': 3 * B * N * H * D * 2 + 4 * B * H * N}
+    dom = max((k for k in kernels if kernels[k]['contractions']), key=lambda k: kernels[k]['ms'])
+    achieved = kernels[dom]['tflops']
+    roofline = {'bound': 'mfma', 'kernel': dom, 'achieved': achieved, 'peak': PEAK_BF16_TFLOPS, 'unit': 'TFLOP/s',
+                'frac': round(achieved / PEAK_BF16_TFLOPS, 4), 'traffic': None,
+                'launch_ms': kernels[dom]['ms'],
+                'flops_per_launch': kernels[dom]['contractions'] * unit}
+
+    total_flops = 9 * unit          # 18*D*B*H*P
+    value = total_flops / step_s / 1e12
+    result = {
+        'metric': 'fwd+bwd TFLOP/s, bf16 2-simplicial attn N=%d w1=%d w2=%d' % (N, w1, w2),
+        'value': round(value, 2), 'unit': 'TFLOP/s', 'n_gpus': 1, 'steps': args.steps, 'warmup': args.warmup,
+        'ms_per_step': round(step_s * 1e3, 3), 'higher_is_better': True, 'scaling': 'weak', 'vs_baseline': None,
+        'dtype': 'bf16', 'data': 'synthetic',
+        'config': {'workload': args.workload, 'batch': B, 'heads': H, 'kv_heads': HK, 'seq_len': N, 'dim_head': D,
+                   'w1': w1, 'w2': w2},
+        'frac_of_bf16_peak': round(value / PEAK_BF16_TFLOPS, 4),
+        'tokens_per_s': round(B * N / step_s, 1),
+        'fwd': {'ms': round(fwd_s * 1e3, 3), 'tflops': round(2 * unit / fwd_s / 1e12, 2),
+                'frac_of_bf16_peak': round(2 * unit / fwd_s / 1e12 / PEAK_BF16_TFLOPS, 4),
+                'tokens_per_s': round(B * N / fwd_s, 1),
+                'hbm_gbs_algorithmic': round(hbm_bytes['fwd'] / (kernels['fwd']['ms'] * 1e-3) / 1e9, 1)},
+        'kernels': kernels,
+        'roofline': roofline,
+    }
+    if args.cpu_slices > 0:
+        result['cpu_baseline'] = cpu_baseline(N, D, w1, w2, args.cpu_slices)
+    print(json.dumps(result))
+
+
+if __name__ == '__main__':
+    main()

@@ -85,16 +85,21 @@ int sa2_supported(int32_t dim_head, int32_t w1, int32_t w2, int32_t dtype);
 
 /* Forward.  Replaces the launch of two_simplicial_attn_fwd_kernel
  * (triton_two_simplicial_attention.py:749-798; kernel :58-228).
- * Writes out (same layout as q) and lse[b,h,n] = log sum exp of the scaled logits. */
+ * Writes out (same layout as q) and lse[b,h,n] = log sum exp of the scaled logits.
+ * out_residual may be NULL; if given (same shape/dtype as out) it receives
+ * bf16(out_fp32 - out), so that out + out_residual carries the fp32 accumulator to
+ * about 16 mantissa bits.  The backward uses it to form delta without the rounding
+ * error of the bf16 output (the reference forms delta from the rounded output, :282). */
 int sa2_fwd(const sa2_problem *prob,
             const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
             const sa2_tensor *v1, const sa2_tensor *v2,
-            const sa2_tensor *out, float *lse, void *hip_stream);
+            const sa2_tensor *out, const sa2_tensor *out_residual, float *lse, void *hip_stream);
 
-/* delta[b,h,n] = sum_d out * dout.  Replaces backward_preprocess_do_o_dot
+/* delta[b,h,n] = sum_d (out + out_residual) * dout; out_residual may be NULL.
+ * Replaces backward_preprocess_do_o_dot
  * (triton_two_simplicial_attention.py:834-849; kernel :230-286). */
-int sa2_bwd_delta(const sa2_problem *prob, const sa2_tensor *out, const sa2_tensor *dout,
-                  float *delta, void *hip_stream);
+int sa2_bwd_delta(const sa2_problem *prob, const sa2_tensor *out, const sa2_tensor *out_residual,
+                  const sa2_tensor *dout, float *delta, void *hip_stream);
 
 /* dQ.  Replaces the dQ half of two_simplicial_attn_bwd_kv2q_kernel
  * (triton_two_simplicial_attention.py:939-1004; kernel :515-712, dq at :697-699,709). */
@@ -123,12 +128,14 @@ int sa2_bwd_dkv2(const sa2_problem *prob,
 
 /* Whole backward: delta, dQ, dK1/dV1, dK2/dV2 in stream order.  Replaces the body
  * of SlidingTwoSimplicialAttention.backward (triton_two_simplicial_attention.py:808-1006).
- * delta_ws is a caller-owned fp32 (batch, heads, seq) workspace.  Gradients are
+ * delta_ws is a caller-owned fp32 (batch, heads, seq) workspace; out_residual may be
+ * NULL (see sa2_fwd).  Gradients are
  * written in the activation dtype and need no prior zeroing. */
 int sa2_bwd(const sa2_problem *prob,
             const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
             const sa2_tensor *v1, const sa2_tensor *v2,
-            const sa2_tensor *out, const sa2_tensor *dout, const float *lse, float *delta_ws,
+            const sa2_tensor *out, const sa2_tensor *out_residual, const sa2_tensor *dout,
+            const float *lse, float *delta_ws,
             const sa2_tensor *dq, const sa2_tensor *dk1, const sa2_tensor *dk2,
             const sa2_tensor *dv1, const sa2_tensor *dv2, void *hip_stream);
 

@@ -76,9 +76,9 @@ def load() -> ctypes.CDLL:
         lib.sa2_supported.restype = ctypes.c_int
         lib.sa2_supported.argtypes = [ctypes.c_int32] * 4
         lib.sa2_fwd.restype = ctypes.c_int
-        lib.sa2_fwd.argtypes = [P, T, T, T, T, T, T, F, V]
+        lib.sa2_fwd.argtypes = [P, T, T, T, T, T, T, T, F, V]
         lib.sa2_bwd_delta.restype = ctypes.c_int
-        lib.sa2_bwd_delta.argtypes = [P, T, T, F, V]
+        lib.sa2_bwd_delta.argtypes = [P, T, T, T, F, V]
         lib.sa2_bwd_dq.restype = ctypes.c_int
         lib.sa2_bwd_dq.argtypes = [P, T, T, T, T, T, T, F, F, T, V]
         lib.sa2_bwd_dkv1.restype = ctypes.c_int
@@ -86,7 +86,7 @@ def load() -> ctypes.CDLL:
         lib.sa2_bwd_dkv2.restype = ctypes.c_int
         lib.sa2_bwd_dkv2.argtypes = [P, T, T, T, T, T, T, F, F, T, T, V]
         lib.sa2_bwd.restype = ctypes.c_int
-        lib.sa2_bwd.argtypes = [P, T, T, T, T, T, T, T, F, F, T, T, T, T, T, V]
+        lib.sa2_bwd.argtypes = [P, T, T, T, T, T, T, T, T, F, F, T, T, T, T, T, V]
         _lib = lib
         return lib
 

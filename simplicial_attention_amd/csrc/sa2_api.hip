@@ -98,8 +98,10 @@ int sa2_supported(int32_t dim_head, int32_t w1, int32_t w2, int32_t dtype) {
 }
 
 int sa2_fwd(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
-            const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *out, float *lse, void *hip_stream) {
+            const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *out, const sa2_tensor *out_residual,
+            float *lse, void *hip_stream) {
     SA2_TRY(check_problem(prob));
+    if (out_residual) SA2_TRY(check_tensor(out_residual, "out_residual"));
     SA2_TRY(check_tensor(q, "q"));
     SA2_TRY(check_tensor(k1, "k1"));
     SA2_TRY(check_tensor(k2, "k2"));
@@ -114,6 +116,7 @@ int sa2_fwd(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, 
     k.v1 = dev(v1);
     k.v2 = dev(v2);
     k.o = dev(out);
+    if (out_residual) k.o_lo = dev(out_residual);
     k.lse = lse;
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
     int grid = prob->batch * prob->heads * ((prob->seq_len + 127) / 128);
@@ -124,14 +127,16 @@ int sa2_fwd(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, 
     return after_launch("forward");
 }
 
-int sa2_bwd_delta(const sa2_problem *prob, const sa2_tensor *out, const sa2_tensor *dout, float *delta,
-                  void *hip_stream) {
+int sa2_bwd_delta(const sa2_problem *prob, const sa2_tensor *out, const sa2_tensor *out_residual,
+                  const sa2_tensor *dout, float *delta, void *hip_stream) {
     SA2_TRY(check_problem(prob));
+    if (out_residual) SA2_TRY(check_tensor(out_residual, "out_residual"));
     SA2_TRY(check_tensor(out, "out"));
     SA2_TRY(check_tensor(dout, "dout"));
     if (!delta) return fail(SA2_ERR_NULL_POINTER, "delta is NULL");
     sa2::KParams k = base_params(prob);
     k.o = dev(out);
+    if (out_residual) k.o_lo = dev(out_residual);
     k.dout = dev(dout);
     k.delta = delta;
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
@@ -223,10 +228,10 @@ int sa2_bwd_dkv2(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor 
 }
 
 int sa2_bwd(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
-            const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *out, const sa2_tensor *dout,
-            const float *lse, float *delta_ws, const sa2_tensor *dq, const sa2_tensor *dk1, const sa2_tensor *dk2,
+            const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *out, const sa2_tensor *out_residual,
+            const sa2_tensor *dout, const float *lse, float *delta_ws, const sa2_tensor *dq, const sa2_tensor *dk1, const sa2_tensor *dk2,
             const sa2_tensor *dv1, const sa2_tensor *dv2, void *hip_stream) {
-    SA2_TRY(sa2_bwd_delta(prob, out, dout, delta_ws, hip_stream));
+    SA2_TRY(sa2_bwd_delta(prob, out, out_residual, dout, delta_ws, hip_stream));
     SA2_TRY(sa2_bwd_dq(prob, q, k1, k2, v1, v2, dout, lse, delta_ws, dq, hip_stream));
     SA2_TRY(sa2_bwd_dkv1(prob, q, k1, k2, v1, v2, dout, lse, delta_ws, dk1, dv1, hip_stream));
     SA2_TRY(sa2_bwd_dkv2(prob, q, k1, k2, v1, v2, dout, lse, delta_ws, dk2, dv2, hip_stream));

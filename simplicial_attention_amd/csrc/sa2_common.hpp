@@ -31,6 +31,7 @@ struct DevTensor {
 
 struct KParams {
     DevTensor q, k1, k2, v1, v2, o, dout, dq, dk1, dk2, dv1, dv2;
+    DevTensor o_lo;       // optional bf16 residual out_fp32 - bf16(out); ptr == nullptr if absent
     float *lse;
     float *delta;
     int B, N, H, HK, G;   // G = H / HK query heads per key/value head
@@ -88,6 +89,92 @@ __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_ex
 // 8h+4a+c, so that the 8 rows a C-layout lane of half h owns are contiguous.
 __device__ __forceinline__ int kslot_pos(int j) {
     return (j & ~15) | ((j & 4) << 1) | ((j & 8) >> 1) | (j & 3);
+}
+
+// d index (within a 32-wide d tile) handled by MFMA row c of a "transposed output"
+// GEMM (output rows = d), chosen so that the 16 accumulator registers of a lane
+// cover 16 consecutive d:  register r of half hf  <->  d = 16*hf + r.
+__device__ __forceinline__ int dmap_row(int c) { return 16 * ((c >> 2) & 1) + 4 * (c >> 3) + (c & 3); }
+
+// ---- LDS staging of a 128-row chunk of a (seq, dim) matrix, 256 threads ----------
+constexpr int kChunkTiles = 4;                       // 32-row tiles per chunk (= waves)
+constexpr int kChunkRows = kChunkTiles * 32;
+constexpr int kChunkPitchT = (kChunkRows + 8) * 2;   // pitch of a transposed chunk row
+__host__ __device__ constexpr int row_pitch(int d) { return (d + 8) * 2; }  // padded row-major pitch
+
+// Row-major copy: dst[row][d], rows row0 .. row0+127 of src; rows >= N are zero.
+template <int D>
+__device__ __forceinline__ void stage_rows(char *dst, const char *src, int64_t sn, int row0, int N) {
+    constexpr int PPR = D / 8;  // 16-byte pieces per row
+    const int tid = threadIdx.x;
+#pragma unroll
+    for (int it = 0; it < kChunkRows * PPR / 256; ++it) {
+        int idx = it * 256 + tid;
+        int row = idx / PPR, piece = idx % PPR;
+        int j = row0 + row;
+        u32x4 v = {0u, 0u, 0u, 0u};
+        if (j < N) v = ld_global16(src + (int64_t)j * sn + piece * 16);
+        *reinterpret_cast<u32x4 *>(dst + row * row_pitch(D) + piece * 16) = v;
+    }
+}
+
+// Transposed copy: dst[d][kslot_pos(row)], so that a lane of half hf reads the 8 rows
+// it needs for one k-step (16 rows) of a GEMM contracting over rows as one 16-byte word.
+template <int D>
+__device__ __forceinline__ void stage_rows_transposed(char *dst, const char *src, int64_t sn, int row0, int N) {
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    constexpr int LPR = D / 2;     // lanes covering one row with 4-byte loads
+    constexpr int GPW = 64 / LPR;  // 4-row groups per wave instruction
+    const int dpair = lane % LPR;
+#pragma unroll
+    for (int it = 0; it < 8 / GPW; ++it) {
+        int rl0 = 32 * wave + 4 * (it * GPW + lane / LPR);
+        uint32_t w[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            int j = row0 + rl0 + r;
+            w[r] = (j < N) ? *reinterpret_cast<const uint32_t *>(src + (int64_t)j * sn + dpair * 4) : 0u;
+        }
+        u32x2 lo = {(w[0] & 0xffffu) | (w[1] << 16), (w[2] & 0xffffu) | (w[3] << 16)};
+        u32x2 hi = {(w[0] >> 16) | (w[1] & 0xffff0000u), (w[2] >> 16) | (w[3] & 0xffff0000u)};
+        int pos = kslot_pos(rl0);
+        *reinterpret_cast<u32x2 *>(dst + (2 * dpair) * kChunkPitchT + pos * 2) = lo;
+        *reinterpret_cast<u32x2 *>(dst + (2 * dpair + 1) * kChunkPitchT + pos * 2) = hi;
+    }
+}
+
+// acc[dt][r] += x[32*dt + 16*hf + r] * g[dt][r]; xrow points at element 16*hf of the row
+template <int DT>
+__device__ __forceinline__ void fma_row(f32x16 (&acc)[DT], const f32x16 (&g)[DT], const char *xrow) {
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+        u32x4 xa = ld_global16(xrow + dt * 64);
+        u32x4 xb = ld_global16(xrow + dt * 64 + 16);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            acc[dt][2 * w] += bf16_lo(xa[w]) * g[dt][2 * w];
+            acc[dt][2 * w + 1] += bf16_hi(xa[w]) * g[dt][2 * w + 1];
+            acc[dt][8 + 2 * w] += bf16_lo(xb[w]) * g[dt][8 + 2 * w];
+            acc[dt][8 + 2 * w + 1] += bf16_hi(xb[w]) * g[dt][8 + 2 * w + 1];
+        }
+    }
+}
+
+// store acc[dt][r] * s as bf16 at d = 32*dt + 16*hf + r; orow points at element 16*hf
+template <int DT>
+__device__ __forceinline__ void store_row(char *orow, const f32x16 (&acc)[DT], float s) {
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) {
+        u32x4 oa, ob;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            oa[w] = pack_bf16(acc[dt][2 * w] * s, acc[dt][2 * w + 1] * s);
+            ob[w] = pack_bf16(acc[dt][8 + 2 * w] * s, acc[dt][8 + 2 * w + 1] * s);
+        }
+        st_global16(orow + dt * 64, oa);
+        st_global16(orow + dt * 64 + 16, ob);
+    }
 }
 
 // Grid index -> logical work item such that the eight XCDs (which receive

@@ -27,54 +27,12 @@ template <int D>
 struct FwdCfg {
     static constexpr int KS = D / 16;          // k-steps of the logit GEMM
     static constexpr int DT = D / 32;          // 32-wide d tiles of the value GEMM
-    static constexpr int CT = 4;               // 32-row tiles per staged chunk (= waves)
-    static constexpr int CR = CT * 32;         // rows per chunk
-    static constexpr int PK = (D + 8) * 2;     // LDS pitch of a K1 row, bytes
-    static constexpr int PV = (CR + 8) * 2;    // LDS pitch of a V1^T row, bytes
-    static constexpr int K1_BYTES = CR * PK;
+    static constexpr int CT = kChunkTiles;     // 32-row tiles per staged chunk (= waves)
+    static constexpr int PK = row_pitch(D);    // LDS pitch of a K1 row, bytes
+    static constexpr int PV = kChunkPitchT;    // LDS pitch of a V1^T row, bytes
+    static constexpr int K1_BYTES = kChunkRows * PK;
     static constexpr int V1T_BYTES = D * PV;
 };
-
-// Stage rows [row0, row0+128) of K1 (row-major) and of V1 (transposed, k-slot order).
-template <int D>
-__device__ __forceinline__ void stage_k1_v1t(char *k1s, char *v1t, const char *k1g, const char *v1g,
-                                             int64_t k1_sn, int64_t v1_sn, int row0, int N) {
-    using C = FwdCfg<D>;
-    const int tid = threadIdx.x;
-    constexpr int PPR = D / 8;  // 16-byte pieces per row
-#pragma unroll
-    for (int it = 0; it < C::CR * PPR / 256; ++it) {
-        int idx = it * 256 + tid;
-        int row = idx / PPR, piece = idx % PPR;
-        int j = row0 + row;
-        u32x4 v = {0u, 0u, 0u, 0u};
-        if (j < N) v = ld_global16(k1g + (int64_t)j * k1_sn + piece * 16);
-        *reinterpret_cast<u32x4 *>(k1s + row * C::PK + piece * 16) = v;
-    }
-    const int wave = tid >> 6, lane = tid & 63;
-    constexpr int LPR = D / 2;        // lanes covering one row with 4-byte loads
-    constexpr int GPW = 64 / LPR;     // 4-row groups per wave instruction
-    const int dpair = lane % LPR;
-#pragma unroll
-    for (int it = 0; it < 8 / GPW; ++it) {
-        int rl0 = 32 * wave + 4 * (it * GPW + lane / LPR);
-        uint32_t w[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            int j = row0 + rl0 + r;
-            w[r] = (j < N) ? *reinterpret_cast<const uint32_t *>(v1g + (int64_t)j * v1_sn + dpair * 4) : 0u;
-        }
-        u32x2 lo = {(w[0] & 0xffffu) | (w[1] << 16), (w[2] & 0xffffu) | (w[3] << 16)};
-        u32x2 hi = {(w[0] >> 16) | (w[1] & 0xffff0000u), (w[2] >> 16) | (w[3] & 0xffff0000u)};
-        int pos = kslot_pos(rl0);
-        *reinterpret_cast<u32x2 *>(v1t + (2 * dpair) * C::PV + pos * 2) = lo;
-        *reinterpret_cast<u32x2 *>(v1t + (2 * dpair + 1) * C::PV + pos * 2) = hi;
-    }
-}
-
-// d index (within a 32-wide d tile) handled by MFMA row c of the value GEMM, chosen
-// so that the 16 accumulator registers of a lane cover 16 consecutive d.
-__device__ __forceinline__ int dmap_row(int c) { return 16 * ((c >> 2) & 1) + 4 * (c >> 3) + (c & 3); }
 
 template <int D>
 __global__ __launch_bounds__(256, 2) void fwd_kernel(KParams p) {
@@ -124,7 +82,8 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(KParams p) {
 
     for (int ct0 = t_begin; ct0 <= t_end; ct0 += C::CT) {
         __syncthreads();
-        stage_k1_v1t<D>(k1s, v1t, k1g, v1g, p.k1.sn, p.v1.sn, ct0 * 32, N);
+        stage_rows<D>(k1s, k1g, p.k1.sn, ct0 * 32, N);
+        stage_rows_transposed<D>(v1t, v1g, p.v1.sn, ct0 * 32, N);
         __syncthreads();
         const int tl = ct0 > wt_lo ? ct0 : wt_lo;
         const int th = (ct0 + C::CT - 1 < wt_hi) ? ct0 + C::CT - 1 : wt_hi;
@@ -214,16 +173,25 @@ __global__ __launch_bounds__(256, 2) void fwd_kernel(KParams p) {
     const float l_tot = l + other_half(l);
     const float inv = 1.f / l_tot;
     char *orow = p.o.ptr + b * p.o.sb + (int64_t)i * p.o.sn + h * p.o.sh + 16 * hf * 2;
+    char *rrow = p.o_lo.ptr ? p.o_lo.ptr + b * p.o_lo.sb + (int64_t)i * p.o_lo.sn + h * p.o_lo.sh + 16 * hf * 2 : nullptr;
 #pragma unroll
     for (int dt = 0; dt < C::DT; ++dt) {
-        u32x4 oa, ob;
+        u32x4 oa, ob, ra, rb;
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
-            oa[w] = pack_bf16(acc[dt][2 * w] * inv, acc[dt][2 * w + 1] * inv);
-            ob[w] = pack_bf16(acc[dt][8 + 2 * w] * inv, acc[dt][8 + 2 * w + 1] * inv);
+            const float x0 = acc[dt][2 * w] * inv, x1 = acc[dt][2 * w + 1] * inv;
+            const float y0 = acc[dt][8 + 2 * w] * inv, y1 = acc[dt][8 + 2 * w + 1] * inv;
+            oa[w] = pack_bf16(x0, x1);
+            ob[w] = pack_bf16(y0, y1);
+            ra[w] = pack_bf16(x0 - bf16_lo(oa[w]), x1 - bf16_hi(oa[w]));
+            rb[w] = pack_bf16(y0 - bf16_lo(ob[w]), y1 - bf16_hi(ob[w]));
         }
         st_global16(orow + dt * 64, oa);
         st_global16(orow + dt * 64 + 16, ob);
+        if (rrow) {
+            st_global16(rrow + dt * 64, ra);
+            st_global16(rrow + dt * 64 + 16, rb);
+        }
     }
     if (hf == 0) p.lse[((int64_t)b * p.H + h) * N + i] = (m + __builtin_amdgcn_logf(l_tot)) * kLn2;
 }

@@ -65,17 +65,21 @@ class SlidingTwoSimplicialAttention(Function):
         scale = dim ** -0.5
         out = torch.empty((batch, seq_len, heads, dim), dtype=q.dtype, device=q.device)
         lse = torch.empty((batch, heads, seq_len), dtype=torch.float32, device=q.device)
+        # bf16 residual of the fp32 accumulator, kept only when a backward may follow
+        needs_grad = any(ctx.needs_input_grad[:5])
+        residual = torch.empty_like(out) if needs_grad else None
         prob = _native.problem(batch, seq_len, heads, kv_heads, dim, w1, w2, True, scale)
         with torch.cuda.device_of(q):
             _native.check(lib.sa2_fwd(prob, *(_native.tensor_arg(t) for t in (q, k1, k2, v1, v2, out)),
+                                      _native.tensor_arg(residual) if needs_grad else None,
                                       lse.data_ptr(), _stream_handle(q.device)))
-        ctx.save_for_backward(q, k1, k2, v1, v2, out, lse)
+        ctx.save_for_backward(q, k1, k2, v1, v2, out, lse, residual)
         ctx.problem = (batch, seq_len, heads, kv_heads, dim, w1, w2, scale)
         return out
 
     @staticmethod
     def backward(ctx, dout):
-        q, k1, k2, v1, v2, out, lse = ctx.saved_tensors
+        q, k1, k2, v1, v2, out, lse, residual = ctx.saved_tensors
         batch, seq_len, heads, kv_heads, dim, w1, w2, scale = ctx.problem
         dout = _unit_inner_stride(dout)
         lib = _native.load()
@@ -85,7 +89,8 @@ class SlidingTwoSimplicialAttention(Function):
         prob = _native.problem(batch, seq_len, heads, kv_heads, dim, w1, w2, True, scale)
         arg = _native.tensor_arg
         with torch.cuda.device_of(q):
-            _native.check(lib.sa2_bwd(prob, arg(q), arg(k1), arg(k2), arg(v1), arg(v2), arg(out), arg(dout),
+            _native.check(lib.sa2_bwd(prob, arg(q), arg(k1), arg(k2), arg(v1), arg(v2), arg(out),
+                                      arg(residual) if residual is not None else None, arg(dout),
                                       lse.data_ptr(), delta.data_ptr(),
                                       arg(dq), arg(dk1), arg(dk2), arg(dv1), arg(dv2), _stream_handle(q.device)))
         return dq, dk1, dk2, dv1, dv2, None, None, None

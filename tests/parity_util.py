@@ -1,0 +1,62 @@
+"""Shared helpers of the GPU parity tests: seeded inputs, oracle calls and the
+tolerance of the build target (|x - ref| <= 2e-2 + 1e-2 |ref| for bf16 against the
+fp32 oracle evaluated on the same bf16-rounded inputs)."""
+import torch
+
+from oracle import reference_attend as R
+
+ATOL, RTOL = 2e-2, 1e-2
+NAMES = ('out', 'dq', 'dk1', 'dk2', 'dv1', 'dv2')
+
+
+def make_inputs(b, n, hq, hk, d, seed, std=1.0):
+    """Draw fp32 on the CPU in the order q, k1, k2, v1, v2, dout; round to bf16."""
+    g = torch.Generator(device='cpu').manual_seed(seed)
+    q = (torch.randn(b, n, hq, d, generator=g) * std).bfloat16()
+    k1, k2, v1, v2 = [(torch.randn(b, n, hk, d, generator=g) * std).bfloat16() for _ in range(4)]
+    dout = torch.randn(b, n, hq, d, generator=g).bfloat16()
+    return q, k1, k2, v1, v2, dout
+
+
+def oracle_fwd_bwd(q, k1, k2, v1, v2, dout, w1, w2, device='cpu', dtype=torch.float32, chunk=64):
+    """fp32 banded oracle on the bf16-rounded values; grouped heads are expanded in
+    '(h g)' order and key/value gradients summed back over the group."""
+    hq, hk = q.shape[2], k1.shape[2]
+    g = hq // hk
+    f = lambda t: t.to(device=device, dtype=dtype)
+    qe = f(q)
+    ke = [R.expand_kv_heads(f(t), g) for t in (k1, k2, v1, v2)]
+    out, lse, grads = R.windowed_banded_fwd_bwd(qe, *ke, f(dout), w1, w2, chunk=chunk)
+    dq, rest = grads[0], grads[1:]
+    rest = [t.unflatten(2, (hk, g)).sum(3) for t in rest]
+    return out, lse, (dq, *rest)
+
+
+def hip_fwd_bwd(q, k1, k2, v1, v2, dout, w1, w2):
+    from simplicial_attention_amd import sliding_two_simplicial_attn
+    ts = [t.cuda().requires_grad_(True) for t in (q, k1, k2, v1, v2)]
+    out = sliding_two_simplicial_attn(ts[0], (ts[1], ts[2]), (ts[3], ts[4]), w1=w1, w2=w2, causal=True)
+    grads = torch.autograd.grad(out, ts, dout.cuda())
+    torch.cuda.synchronize()
+    return out.detach(), grads
+
+
+def compare(name, got, ref):
+    got = got.detach().float().cpu()
+    ref = ref.detach().float().cpu()
+    err = (got - ref).abs()
+    bad = int((err > ATOL + RTOL * ref.abs()).sum())
+    rel_f = float(err.norm() / ref.norm().clamp_min(1e-30))
+    return dict(name=name, max_abs=float(err.max()), ref_max=float(ref.abs().max()), rel_fro=rel_f, bad=bad)
+
+
+def check_all(got_out, got_grads, ref_out, ref_grads, rel_fro_limit=2e-2, verbose=True):
+    rows = [compare(n, g, r) for n, g, r in zip(NAMES, (got_out, *got_grads), (ref_out, *ref_grads))]
+    if verbose:
+        for r in rows:
+            print('   %-4s max_abs %.3e  ref_max %.3e  rel_fro %.3e  out_of_tol %d' %
+                  (r['name'], r['max_abs'], r['ref_max'], r['rel_fro'], r['bad']), flush=True)
+    for r in rows:
+        assert r['bad'] == 0, f"{r['name']}: {r['bad']} elements outside |x-ref| <= {ATOL} + {RTOL}|ref| (max abs {r['max_abs']:.3e})"
+        assert r['rel_fro'] <= rel_fro_limit, f"{r['name']}: relative Frobenius error {r['rel_fro']:.3e} > {rel_fro_limit}"
+    return rows
