@@ -1,0 +1,161 @@
+"""CPU-side checks: the C-ABI library loads, exports every symbol that include/sa2.h
+declares, validates its arguments before touching a device; the Python front end
+keeps the reference's names, defaults, parameter names and error behaviour."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from simplicial_attention_amd import _native
+import simplicial_attention_amd as S
+from oracle import reference_attend as R
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.fixture(scope='module')
+def lib():
+    if not os.path.exists(_native.LIB_PATH):
+        _native.build()
+    return _native.load()
+
+
+def header_symbols():
+    text = open(os.path.join(ROOT, 'include', 'sa2.h')).read()
+    text = re.sub(r'/\*.*?\*/', '', text, flags=re.S)
+    return sorted(set(re.findall(r'\b(sa2_[a-z0-9_]+)\s*\(', text)))
+
+
+def test_every_declared_symbol_is_exported(lib):
+    names = header_symbols()
+    assert set(names) == set(_native.EXPORTS)
+    for name in names:
+        assert getattr(lib, name) is not None
+    assert lib.sa2_version() == 100
+
+
+def test_supported_matrix(lib):
+    assert lib.sa2_supported(64, 512, 32, 0) == 1
+    assert lib.sa2_supported(128, 512, 64, 0) == 1
+    assert lib.sa2_supported(32, 512, 32, 0) == 0
+    assert lib.sa2_supported(128, 0, 32, 0) == 0
+    assert lib.sa2_supported(128, 512, 32, 1) == 0
+
+
+def _dummy(ptr=0x1000, sb=1024, sn=128, sh=8):
+    return _native.TensorArg(ptr, sb, sn, sh)
+
+
+def test_argument_validation_happens_before_any_launch(lib):
+    good = _native.problem(1, 64, 2, 1, 128, 512, 32, True, 128 ** -0.5)
+    t = _dummy()
+    lse = ctypes.c_void_p(0x2000)
+
+    def fwd(prob, *tensors, lse_ptr=lse):
+        return lib.sa2_fwd(prob, *tensors, None, lse_ptr, None)
+
+    assert fwd(None, t, t, t, t, t, t) == 1
+    assert fwd(good, None, t, t, t, t, t) == 1
+    assert b'q' in lib.sa2_last_error()
+    assert fwd(good, t, t, t, t, t, t, lse_ptr=None) == 1
+    for field, value, code in [('dim_head', 96, 3), ('causal', 0, 3), ('dtype', 7, 3), ('w1', 0, 2), ('w2', -1, 2),
+                               ('seq_len', 0, 2), ('kv_heads', 3, 2), ('batch', 0, 2)]:
+        bad = _native.problem(1, 64, 2, 1, 128, 512, 32, True, 128 ** -0.5)
+        setattr(bad, field, value)
+        assert fwd(bad, t, t, t, t, t, t) == code, field
+        assert lib.sa2_last_error() != b''
+    assert fwd(good, _dummy(ptr=0x1008), t, t, t, t, t) == 4
+    assert fwd(good, t, _dummy(sn=132), t, t, t, t) == 4
+    with pytest.raises(_native.Sa2Error) as e:
+        _native.check(fwd(good, t, t, _dummy(sh=4), t, t, t))
+    assert 'SA2_ERR_ALIGNMENT' in str(e.value) and 'k2' in str(e.value)
+    # backward entry points validate the same way
+    assert lib.sa2_bwd_delta(good, None, None, t, lse, None) == 1
+    assert lib.sa2_bwd_dq(good, t, t, t, t, t, t, None, lse, t, None) == 1
+    assert lib.sa2_bwd_dkv1(good, t, t, t, t, t, t, lse, lse, None, t, None) == 1
+    assert lib.sa2_bwd_dkv2(good, t, t, t, t, t, t, lse, lse, t, _dummy(ptr=0x1004), None) == 4
+    assert lib.sa2_bwd(good, t, t, t, t, t, None, None, t, lse, lse, t, t, t, t, t, None) == 1
+
+
+def test_function_rejects_what_the_kernels_do_not_cover():
+    q = torch.randn(1, 16, 2, 64)
+    with pytest.raises(AssertionError):          # reference: assert all is_cuda (triton_two_simplicial_attention.py:729)
+        S.sliding_two_simplicial_attn(q, (q, q), (q, q))
+    with pytest.raises(AssertionError):
+        S.sliding_two_simplicial_attn(q, (q,), (q, q))
+    with pytest.raises(AssertionError):          # head divisibility (triton_two_simplicial_attention.py:1030)
+        S.sliding_two_simplicial_attn(torch.randn(1, 16, 3, 64), (q, q), (q, q))
+
+
+def test_module_mirrors_reference_constructor_and_parameters():
+    m = S.SlidingWindowTwoSimplicialMHA(dim=512, dim_head=64, heads=8)
+    sd = m.state_dict()
+    assert set(sd) == {'q_norm.weight', 'k_norms.0.weight', 'k_norms.1.weight', 'v_norms.0.weight',
+                       'v_norms.1.weight', 'to_qkv.weight', 'combine_heads.weight'}
+    assert sd['to_qkv.weight'].shape == (8 * 64 + 2 * 8 * 64 + 2 * 8 * 64, 512)
+    assert sd['combine_heads.weight'].shape == (512, 512)
+    assert m.attend.keywords == {'w1': 512, 'w2': 32, 'causal': True}
+    g = S.SlidingWindowTwoSimplicialMHA(dim=256, dim_head=64, heads=8, key_value_heads=4, w1=128, w2=16,
+                                        prenorm=True, postnorm=True, qk_rmsnorm=False)
+    assert g.to_qkv.weight.shape == (8 * 64 + 2 * 4 * 64 + 2 * 4 * 64, 256)
+    assert {'prenorm.weight', 'postnorm.weight'} <= set(g.state_dict())
+    assert g.query_head_groups == 2
+    with pytest.raises(AssertionError):
+        S.SlidingWindowTwoSimplicialMHA(dim=64, number_key_value_sets=3)
+    with pytest.raises(AssertionError):
+        S.SlidingWindowTwoSimplicialMHA(dim=64, head_first_dim=True)
+    with pytest.raises(AssertionError):
+        S.TwoSimplicialMHA(dim=64, number_key_value_sets=2)
+
+
+def test_alias_module_exposes_reference_names():
+    from simplicial_attention_amd import triton_two_simplicial_attention as T
+    assert T.sliding_two_simplicial_attn is S.sliding_two_simplicial_attn
+    assert T.SlidingWindowTwoSimplicialMHA is S.SlidingWindowTwoSimplicialMHA
+    assert T._sliding_two_simplicial_attn.__self__ is S.SlidingTwoSimplicialAttention
+
+
+def test_module_channel_order_with_oracle_attend():
+    """Module plumbing (projection split, '(head, set, d)' channel order, per-head
+    RMSNorm on q, k and v, merge) against an explicit restatement with the same weights
+    (simplicial_mha.py:110-138 in the reference), using the oracle as `attend`."""
+    torch.manual_seed(0)
+    dim, heads, kvh, dh, n = 32, 4, 2, 8, 12
+    attend = lambda q, k, v: R.sliding_two_simplicial_attn(q, k, v, w1=5, w2=3)
+    m = S.HigherOrderAttention(dim, dim_head=dh, heads=heads, key_value_heads=kvh, attend=attend, head_first_dim=False)
+    for prm in m.parameters():
+        torch.nn.init.normal_(prm, std=0.5)
+    x = torch.randn(2, n, dim)
+    got = m(x)
+    w = m.to_qkv.weight
+    proj = x @ w.t()
+    q = proj[..., :heads * dh].reshape(2, n, heads, dh)
+    k = proj[..., heads * dh:heads * dh + 2 * kvh * dh].reshape(2, n, kvh, 2, dh)
+    v = proj[..., heads * dh + 2 * kvh * dh:].reshape(2, n, kvh, 2, dh)
+    rms = lambda t, wt: t / t.pow(2).mean(-1, keepdim=True).add(torch.finfo(t.dtype).eps).sqrt() * wt
+    q = rms(q, m.q_norm.weight)
+    k1, k2 = rms(k[..., 0, :], m.k_norms[0].weight), rms(k[..., 1, :], m.k_norms[1].weight)
+    v1, v2 = rms(v[..., 0, :], m.v_norms[0].weight), rms(v[..., 1, :], m.v_norms[1].weight)
+    out = R.sliding_two_simplicial_attn(q, (k1, k2), (v1, v2), w1=5, w2=3)
+    want = out.reshape(2, n, heads * dh) @ m.combine_heads.weight.t()
+    assert torch.allclose(got, want, atol=1e-5)
+
+
+def test_naive_attend_matches_oracle_restatement():
+    g = torch.Generator().manual_seed(1)
+    q = torch.randn(2, 4, 10, 8, generator=g)
+    k1, k2, v1, v2 = [torch.randn(2, 2, 10, 8, generator=g) for _ in range(4)]
+    for causal in (False, True):
+        a = S.naive_two_simplicial_attend(q, (k1, k2), (v1, v2), causal=causal)
+        b = R.naive_two_simplicial_attend(q, (k1, k2), (v1, v2), causal=causal)
+        assert torch.allclose(a, b, atol=1e-6)
+    t = torch.randn(1, 16, 512)
+    assert S.TwoSimplicialMHA(dim=512, causal=True)(t).shape == t.shape   # tests/test_attn.py:49-55 in the reference
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess, sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, 'bench.py'), '--gpus', '2'], capture_output=True, text=True)
+    assert r.returncode != 0 and 'one GPU' in r.stderr
