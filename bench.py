@@ -12,7 +12,8 @@ Algorithmic work (attended triples P per (batch, head), P = sum_i min(i+1,w1) mi
 `value` uses 18*D*B*H*P over the fwd+bwd time.  Each kernel is also timed on its own
 through the C ABI with HIP events on the launch stream; the `roofline` object is for
 the kernel with the longest launch, priced with the contractions that kernel needs
-for its own outputs (fwd 2, dQ 3, dK1/dV1 4, dK2/dV2 4; 2*D flop each per triple).
+for its own outputs (fwd 2: S, O; dQ/dK2/dV2 4: S, dP, G, T; dK1/dV1 4: S, dP, dK1, dV1;
+2*D flop each per triple).
 """
 import argparse
 import json
@@ -70,6 +71,7 @@ def main():
     ap.add_argument('--workload', default='cfg3_raw_kernel_b4_h8_n8192_d128_w512_w32', choices=sorted(WORKLOADS))
     ap.add_argument('--cpu-slices', type=int, default=4, help='(batch, head) slices of the CPU baseline sample (0 = skip)')
     ap.add_argument('--kernel-iters', type=int, default=5, help='launches per kernel for the per-kernel timing')
+    ap.add_argument('--only', default=None, help='time only this kernel through the C ABI (fwd, bwd_delta, bwd_dq_dkv2, bwd_dkv1); for profiling')
     args = ap.parse_args()
     if args.gpus != 1:
         print('bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path exists)', file=sys.stderr)
@@ -101,25 +103,28 @@ def main():
         out = fwd()
         return torch.autograd.grad(out, ins, dout)
 
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    step_s = (time.perf_counter() - t0) / args.steps
-
-    # forward only (same API, no graph kept)
-    with torch.no_grad():
-        for _ in range(2):
-            fwd()
+    step_s = fwd_s = float('nan')
+    if args.only is None:
+        for _ in range(args.warmup):
+            step()
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        for _ in range(max(3, args.steps)):
-            fwd()
+        for _ in range(args.steps):
+            step()
         torch.cuda.synchronize()
-        fwd_s = (time.perf_counter() - t0) / max(3, args.steps)
+        step_s = (time.perf_counter() - t0) / args.steps
+
+    # forward only (same API, no graph kept)
+    if args.only is None:
+        with torch.no_grad():
+            for _ in range(2):
+                fwd()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(max(3, args.steps)):
+                fwd()
+            torch.cuda.synchronize()
+            fwd_s = (time.perf_counter() - t0) / max(3, args.steps)
 
     # ---- per-kernel timing through the C ABI, HIP events on the launch stream
     P = attended_triples(N, w1, w2)
@@ -136,14 +141,23 @@ def main():
     dq = torch.empty_like(qd)
     dk1, dk2, dv1, dv2 = (torch.empty_like(k1d) for _ in range(4))
     five = (arg(qd), arg(k1d), arg(k2d), arg(v1d), arg(v2d))
+    ws_bytes = lib.sa2_bwd_workspace_bytes(prob)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
     launches = {
         'fwd': (2, lambda: lib.sa2_fwd(prob, *five, arg(out), arg(res), lse.data_ptr(), sh)),
         'bwd_delta': (0, lambda: lib.sa2_bwd_delta(prob, arg(out), arg(res), arg(dout), delta.data_ptr(), sh)),
-        'bwd_dq': (3, lambda: lib.sa2_bwd_dq(prob, *five, arg(dout), lse.data_ptr(), delta.data_ptr(), arg(dq), sh)),
+        'bwd_dq_dkv2': (4, lambda: lib.sa2_bwd_dq_dkv2(prob, *five, arg(dout), lse.data_ptr(), delta.data_ptr(), arg(dq), arg(dk2),
+                                                      arg(dv2), ws.data_ptr(), ws_bytes, sh)),
         'bwd_dkv1': (4, lambda: lib.sa2_bwd_dkv1(prob, *five, arg(dout), lse.data_ptr(), delta.data_ptr(), arg(dk1), arg(dv1), sh)),
-        'bwd_dkv2': (4, lambda: lib.sa2_bwd_dkv2(prob, *five, arg(dout), lse.data_ptr(), delta.data_ptr(), arg(dk2), arg(dv2), sh)),
     }
     kernels = {}
+    if args.only is not None:
+        # the later kernels read what the earlier ones wrote: run the chain once, untimed
+        for name, (_, fn) in launches.items():
+            if name == args.only:
+                break
+            _native.check(fn())
+        launches = {args.only: launches[args.only]}
     for name, (ncontr, fn) in launches.items():
         _native.check(fn())
         torch.cuda.synchronize()
@@ -158,6 +172,9 @@ def main():
         ms = statistics.mean(a.elapsed_time(b_) for a, b_ in evs)
         kernels[name] = {'ms': round(ms, 4), 'contractions': ncontr,
                          'tflops': round(ncontr * unit / (ms * 1e-3) / 1e12, 2) if ncontr else None}
+    if args.only is not None:
+        print(json.dumps({'workload': args.workload, 'kernels': kernels}))
+        return
     hbm_bytes = {'fwd': 7 * B * N * H * D * 2 + 4 * B * H * N, 'bwd_delta': 3 * B * N * H * D * 2 + 4 * B * H * N}
     dom = max((k for k in kernels if kernels[k]['contractions']), key=lambda k: kernels[k]['ms'])
     achieved = kernels[dom]['tflops']

@@ -58,7 +58,7 @@ typedef struct sa2_problem {
     int32_t kv_heads;   /* key/value heads, divides heads */
     int32_t dim_head;   /* 64 or 128 */
     int32_t w1;         /* window of the first key/value set  (reference default 512) */
-    int32_t w2;         /* window of the second key/value set (reference default 32)  */
+    int32_t w2;         /* window of the second key/value set (reference default 32), <= 64 */
     int32_t causal;     /* must be 1 */
     float   scale;      /* softmax scale, dim_head^-0.5 in the reference (:735) */
     int32_t dtype;      /* sa2_dtype of the activations */
@@ -78,8 +78,8 @@ int sa2_version(void);
 /* Message of the last failing call on this thread ("" if none). */
 const char *sa2_last_error(void);
 
-/* 1 if the kernels cover this configuration, else 0.  Replaces the silent limits
- * of the reference (HEAD_DIM fixed to 64, w2 <= 32:
+/* 1 if the kernels cover this configuration (dim_head 64 or 128, w2 <= 64, bf16), else 0.
+ * Replaces the silent limits of the reference (HEAD_DIM fixed to 64, w2 <= 32:
  * triton_two_simplicial_attention.py:51,291,508,586). */
 int sa2_supported(int32_t dim_head, int32_t w1, int32_t w2, int32_t dtype);
 
@@ -101,13 +101,23 @@ int sa2_fwd(const sa2_problem *prob,
 int sa2_bwd_delta(const sa2_problem *prob, const sa2_tensor *out, const sa2_tensor *out_residual,
                   const sa2_tensor *dout, float *delta, void *hip_stream);
 
-/* dQ.  Replaces the dQ half of two_simplicial_attn_bwd_kv2q_kernel
- * (triton_two_simplicial_attention.py:939-1004; kernel :515-712, dq at :697-699,709). */
-int sa2_bwd_dq(const sa2_problem *prob,
-               const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
-               const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *dout,
-               const float *lse, const float *delta,
-               const sa2_tensor *dq, void *hip_stream);
+/* Bytes of device workspace the backward needs for this problem (fp32 partial rows of
+ * dK2/dV2, one block per 32-row query tile); -1 if the problem is invalid.  The
+ * reference has no counterpart: its five fp32 gradient buffers of
+ * triton_two_simplicial_attention.py:853-857 play the same role. */
+int64_t sa2_bwd_workspace_bytes(const sa2_problem *prob);
+
+/* dQ, dK2, dV2.  Replaces both passes of two_simplicial_attn_bwd_kv2q_kernel
+ * (triton_two_simplicial_attention.py:938-1004; kernel :515-712; dq :697-699,709;
+ * dk2/dv2 :680-683, :695, :702-707).  One kernel owns the query rows (dQ complete,
+ * dK2/dV2 as partial rows in the workspace), a second one sums the partial rows and
+ * the query heads of a group.  No atomics; results are bitwise reproducible. */
+int sa2_bwd_dq_dkv2(const sa2_problem *prob,
+                    const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
+                    const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *dout,
+                    const float *lse, const float *delta,
+                    const sa2_tensor *dq, const sa2_tensor *dk2, const sa2_tensor *dv2,
+                    void *workspace, int64_t workspace_bytes, void *hip_stream);
 
 /* dK1, dV1 (first key/value set, window w1).  Replaces two_simplicial_attn_bwd_kv1_kernel
  * (triton_two_simplicial_attention.py:868-934; kernel :298-503). */
@@ -117,19 +127,11 @@ int sa2_bwd_dkv1(const sa2_problem *prob,
                  const float *lse, const float *delta,
                  const sa2_tensor *dk1, const sa2_tensor *dv1, void *hip_stream);
 
-/* dK2, dV2 (second key/value set, window w2).  Replaces the dK2/dV2 half of the two
- * passes of two_simplicial_attn_bwd_kv2q_kernel
- * (triton_two_simplicial_attention.py:938-1004; kernel :515-712, :680-683, :695, :702-707). */
-int sa2_bwd_dkv2(const sa2_problem *prob,
-                 const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
-                 const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *dout,
-                 const float *lse, const float *delta,
-                 const sa2_tensor *dk2, const sa2_tensor *dv2, void *hip_stream);
-
 /* Whole backward: delta, dQ, dK1/dV1, dK2/dV2 in stream order.  Replaces the body
  * of SlidingTwoSimplicialAttention.backward (triton_two_simplicial_attention.py:808-1006).
- * delta_ws is a caller-owned fp32 (batch, heads, seq) workspace; out_residual may be
- * NULL (see sa2_fwd).  Gradients are
+ * delta_ws is a caller-owned fp32 (batch, heads, seq) buffer, workspace a caller-owned
+ * buffer of at least sa2_bwd_workspace_bytes() bytes; out_residual may be NULL (see
+ * sa2_fwd).  Gradients are
  * written in the activation dtype and need no prior zeroing. */
 int sa2_bwd(const sa2_problem *prob,
             const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
@@ -137,7 +139,8 @@ int sa2_bwd(const sa2_problem *prob,
             const sa2_tensor *out, const sa2_tensor *out_residual, const sa2_tensor *dout,
             const float *lse, float *delta_ws,
             const sa2_tensor *dq, const sa2_tensor *dk1, const sa2_tensor *dk2,
-            const sa2_tensor *dv1, const sa2_tensor *dv2, void *hip_stream);
+            const sa2_tensor *dv1, const sa2_tensor *dv2,
+            void *workspace, int64_t workspace_bytes, void *hip_stream);
 
 #ifdef __cplusplus
 }

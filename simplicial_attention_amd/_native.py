@@ -25,7 +25,7 @@ STATUS_NAMES = {
 }
 
 EXPORTS = ('sa2_version', 'sa2_last_error', 'sa2_supported', 'sa2_fwd', 'sa2_bwd_delta',
-           'sa2_bwd_dq', 'sa2_bwd_dkv1', 'sa2_bwd_dkv2', 'sa2_bwd')
+           'sa2_bwd_workspace_bytes', 'sa2_bwd_dq_dkv2', 'sa2_bwd_dkv1', 'sa2_bwd')
 
 
 class Sa2Error(RuntimeError):
@@ -79,14 +79,14 @@ def load() -> ctypes.CDLL:
         lib.sa2_fwd.argtypes = [P, T, T, T, T, T, T, T, F, V]
         lib.sa2_bwd_delta.restype = ctypes.c_int
         lib.sa2_bwd_delta.argtypes = [P, T, T, T, F, V]
-        lib.sa2_bwd_dq.restype = ctypes.c_int
-        lib.sa2_bwd_dq.argtypes = [P, T, T, T, T, T, T, F, F, T, V]
+        lib.sa2_bwd_workspace_bytes.restype = ctypes.c_int64
+        lib.sa2_bwd_workspace_bytes.argtypes = [P]
+        lib.sa2_bwd_dq_dkv2.restype = ctypes.c_int
+        lib.sa2_bwd_dq_dkv2.argtypes = [P, T, T, T, T, T, T, F, F, T, T, T, V, ctypes.c_int64, V]
         lib.sa2_bwd_dkv1.restype = ctypes.c_int
         lib.sa2_bwd_dkv1.argtypes = [P, T, T, T, T, T, T, F, F, T, T, V]
-        lib.sa2_bwd_dkv2.restype = ctypes.c_int
-        lib.sa2_bwd_dkv2.argtypes = [P, T, T, T, T, T, T, F, F, T, T, V]
         lib.sa2_bwd.restype = ctypes.c_int
-        lib.sa2_bwd.argtypes = [P, T, T, T, T, T, T, T, T, F, F, T, T, T, T, T, V]
+        lib.sa2_bwd.argtypes = [P, T, T, T, T, T, T, T, T, F, F, T, T, T, T, T, V, ctypes.c_int64, V]
         _lib = lib
         return lib
 

@@ -6,10 +6,14 @@
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
+#include <cstring>
 
 #include "sa2_bwd.hpp"
+#include "sa2_bwd_qk2.hpp"
 #include "sa2_common.hpp"
 #include "sa2_fwd.hpp"
+#include "sa2_fwd_ds.hpp"
 
 namespace {
 
@@ -31,6 +35,7 @@ int check_problem(const sa2_problem *p) {
     if (p->heads % p->kv_heads != 0)
         return fail(SA2_ERR_BAD_SHAPE, "heads=%d is not a multiple of kv_heads=%d", p->heads, p->kv_heads);
     if (p->w1 < 1 || p->w2 < 1) return fail(SA2_ERR_BAD_SHAPE, "windows w1=%d w2=%d must be >= 1", p->w1, p->w2);
+    if (p->w2 > 64) return fail(SA2_ERR_UNSUPPORTED, "w2=%d is not supported (at most 64)", p->w2);
     if (p->causal != 1) return fail(SA2_ERR_UNSUPPORTED, "only causal=1 is defined for the sliding windows");
     if (p->dtype != SA2_BF16) return fail(SA2_ERR_UNSUPPORTED, "dtype %d is not supported (bf16 only)", p->dtype);
     if (p->dim_head != 64 && p->dim_head != 128)
@@ -94,7 +99,7 @@ int sa2_version(void) { return SA2_VERSION; }
 const char *sa2_last_error(void) { return g_err; }
 
 int sa2_supported(int32_t dim_head, int32_t w1, int32_t w2, int32_t dtype) {
-    return (dim_head == 64 || dim_head == 128) && w1 >= 1 && w2 >= 1 && dtype == SA2_BF16;
+    return (dim_head == 64 || dim_head == 128) && w1 >= 1 && w2 >= 1 && w2 <= 64 && dtype == SA2_BF16;
 }
 
 int sa2_fwd(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
@@ -119,11 +124,20 @@ int sa2_fwd(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, 
     if (out_residual) k.o_lo = dev(out_residual);
     k.lse = lse;
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
-    int grid = prob->batch * prob->heads * ((prob->seq_len + 127) / 128);
-    if (prob->dim_head == 128)
-        hipLaunchKernelGGL(sa2::fwd_kernel<128>, dim3(grid), dim3(256), 0, s, k);
-    else
-        hipLaunchKernelGGL(sa2::fwd_kernel<64>, dim3(grid), dim3(256), 0, s, k);
+    const char *impl = std::getenv("SA2_FWD_IMPL");
+    if (impl && std::strcmp(impl, "chunk") == 0) {
+        int grid = prob->batch * prob->heads * ((prob->seq_len + 127) / 128);
+        if (prob->dim_head == 128)
+            hipLaunchKernelGGL(sa2::fwd_kernel<128>, dim3(grid), dim3(256), 0, s, k);
+        else
+            hipLaunchKernelGGL(sa2::fwd_kernel<64>, dim3(grid), dim3(256), 0, s, k);
+    } else {
+        int grid = prob->batch * prob->heads * ((prob->seq_len + 31) / 32);
+        if (prob->dim_head == 128)
+            hipLaunchKernelGGL(sa2::fwd_ds_kernel<128>, dim3(grid), dim3(256), 0, s, k);
+        else
+            hipLaunchKernelGGL(sa2::fwd_ds_kernel<64>, dim3(grid), dim3(256), 0, s, k);
+    }
     return after_launch("forward");
 }
 
@@ -175,20 +189,54 @@ static int bwd_common(const sa2_problem *prob, const sa2_tensor *q, const sa2_te
     return SA2_OK;
 }
 
-int sa2_bwd_dq(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
-               const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *dout, const float *lse,
-               const float *delta, const sa2_tensor *dq, void *hip_stream) {
+// rows of K2/V2 a 32-row query tile can reach: 32 own + (w2max - 1) below it
+static int qk2_w2max(int w2) { return w2 <= 32 ? 32 : 64; }
+
+int64_t sa2_bwd_workspace_bytes(const sa2_problem *prob) {
+    if (check_problem(prob) != SA2_OK) return -1;
+    const int srows = 31 + qk2_w2max(prob->w2);
+    return sa2::qk2_ws_floats(prob->batch, prob->heads, prob->seq_len, prob->dim_head, srows) * 4;
+}
+
+int sa2_bwd_dq_dkv2(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
+                    const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *dout, const float *lse,
+                    const float *delta, const sa2_tensor *dq, const sa2_tensor *dk2, const sa2_tensor *dv2,
+                    void *workspace, int64_t workspace_bytes, void *hip_stream) {
     sa2::KParams k;
     SA2_TRY(bwd_common(prob, q, k1, k2, v1, v2, dout, lse, delta, &k));
     SA2_TRY(check_tensor(dq, "dq"));
+    SA2_TRY(check_tensor(dk2, "dk2"));
+    SA2_TRY(check_tensor(dv2, "dv2"));
+    if (!workspace) return fail(SA2_ERR_NULL_POINTER, "workspace is NULL");
+    if ((reinterpret_cast<uintptr_t>(workspace) & 15) != 0) return fail(SA2_ERR_ALIGNMENT, "workspace must be 16-byte aligned");
+    const int64_t need = sa2_bwd_workspace_bytes(prob);
+    if (workspace_bytes < need)
+        return fail(SA2_ERR_BAD_SHAPE, "workspace of %lld bytes is smaller than the %lld bytes sa2_bwd_workspace_bytes() asks for",
+                    (long long)workspace_bytes, (long long)need);
     k.dq = dev(dq);
+    k.dk2 = dev(dk2);
+    k.dv2 = dev(dv2);
+    float *ws = static_cast<float *>(workspace);
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
-    int grid = prob->batch * prob->heads * ((prob->seq_len + 127) / 128);
-    if (prob->dim_head == 128)
-        hipLaunchKernelGGL(sa2::bwd_dq_kernel<128>, dim3(grid), dim3(256), 0, s, k);
+    const int grid = prob->batch * prob->heads * ((prob->seq_len + 31) / 32);
+    const int w2max = qk2_w2max(prob->w2);
+    if (prob->dim_head == 128 && w2max == 32)
+        hipLaunchKernelGGL((sa2::bwd_qk2_kernel<128, 32>), dim3(grid), dim3(256), 0, s, k, ws);
+    else if (prob->dim_head == 128)
+        hipLaunchKernelGGL((sa2::bwd_qk2_kernel<128, 64>), dim3(grid), dim3(256), 0, s, k, ws);
+    else if (w2max == 32)
+        hipLaunchKernelGGL((sa2::bwd_qk2_kernel<64, 32>), dim3(grid), dim3(256), 0, s, k, ws);
     else
-        hipLaunchKernelGGL(sa2::bwd_dq_kernel<64>, dim3(grid), dim3(256), 0, s, k);
-    return after_launch("dq");
+        hipLaunchKernelGGL((sa2::bwd_qk2_kernel<64, 64>), dim3(grid), dim3(256), 0, s, k, ws);
+    SA2_TRY(after_launch("dq/dk2/dv2"));
+    const int64_t rows = (int64_t)prob->batch * prob->kv_heads * prob->seq_len;
+    const int rows_per_block = 256 / (prob->dim_head / 8);
+    const int cgrid = (int)((rows + rows_per_block - 1) / rows_per_block);
+    if (prob->dim_head == 128)
+        hipLaunchKernelGGL(sa2::dk2_dv2_combine_kernel<128>, dim3(cgrid), dim3(256), 0, s, k, ws, 31 + w2max);
+    else
+        hipLaunchKernelGGL(sa2::dk2_dv2_combine_kernel<64>, dim3(cgrid), dim3(256), 0, s, k, ws, 31 + w2max);
+    return after_launch("dk2/dv2 combine");
 }
 
 int sa2_bwd_dkv1(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
@@ -209,32 +257,15 @@ int sa2_bwd_dkv1(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor 
     return after_launch("dk1/dv1");
 }
 
-int sa2_bwd_dkv2(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
-                 const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *dout, const float *lse,
-                 const float *delta, const sa2_tensor *dk2, const sa2_tensor *dv2, void *hip_stream) {
-    sa2::KParams k;
-    SA2_TRY(bwd_common(prob, q, k1, k2, v1, v2, dout, lse, delta, &k));
-    SA2_TRY(check_tensor(dk2, "dk2"));
-    SA2_TRY(check_tensor(dv2, "dv2"));
-    k.dk2 = dev(dk2);
-    k.dv2 = dev(dv2);
-    hipStream_t s = static_cast<hipStream_t>(hip_stream);
-    int grid = prob->batch * prob->kv_heads * ((prob->seq_len + 127) / 128);
-    if (prob->dim_head == 128)
-        hipLaunchKernelGGL(sa2::bwd_dkv2_kernel<128>, dim3(grid), dim3(256), 0, s, k);
-    else
-        hipLaunchKernelGGL(sa2::bwd_dkv2_kernel<64>, dim3(grid), dim3(256), 0, s, k);
-    return after_launch("dk2/dv2");
-}
-
 int sa2_bwd(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
             const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *out, const sa2_tensor *out_residual,
-            const sa2_tensor *dout, const float *lse, float *delta_ws, const sa2_tensor *dq, const sa2_tensor *dk1, const sa2_tensor *dk2,
-            const sa2_tensor *dv1, const sa2_tensor *dv2, void *hip_stream) {
+            const sa2_tensor *dout, const float *lse, float *delta_ws, const sa2_tensor *dq, const sa2_tensor *dk1,
+            const sa2_tensor *dk2, const sa2_tensor *dv1, const sa2_tensor *dv2, void *workspace,
+            int64_t workspace_bytes, void *hip_stream) {
     SA2_TRY(sa2_bwd_delta(prob, out, out_residual, dout, delta_ws, hip_stream));
-    SA2_TRY(sa2_bwd_dq(prob, q, k1, k2, v1, v2, dout, lse, delta_ws, dq, hip_stream));
+    SA2_TRY(sa2_bwd_dq_dkv2(prob, q, k1, k2, v1, v2, dout, lse, delta_ws, dq, dk2, dv2, workspace, workspace_bytes,
+                            hip_stream));
     SA2_TRY(sa2_bwd_dkv1(prob, q, k1, k2, v1, v2, dout, lse, delta_ws, dk1, dv1, hip_stream));
-    SA2_TRY(sa2_bwd_dkv2(prob, q, k1, k2, v1, v2, dout, lse, delta_ws, dk2, dv2, hip_stream));
     return SA2_OK;
 }
 

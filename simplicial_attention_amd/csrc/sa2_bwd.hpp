@@ -3,12 +3,11 @@
 // The reference computes the backward with two_simplicial_attn_bwd_kv1_kernel and two
 // passes of two_simplicial_attn_bwd_kv2q_kernel
 // (simplicial_attention/triton_two_simplicial_attention.py:298-503, 515-712) plus fp32
-// atomics for a dQ that is later overwritten.  Here the backward is four atomic-free
-// kernels, each of which owns the rows it writes:
-//   delta_kernel     delta_i = sum_d o_i do_i                       (:230-286 there)
-//   bwd_dq_kernel    owns query rows i       -> dQ
-//   bwd_dkv2_kernel  owns rows k of K2/V2    -> dK2, dV2   (query rows i = k + dlt)
-//   bwd_dkv1_kernel  owns rows j of K1/V1    -> dK1, dV1
+// atomics for a dQ that is later overwritten.  Here the backward is atomic-free:
+//   delta_kernel      delta_i = sum_d o_i do_i                      (:230-286 there)
+//   bwd_qk2_kernel    owns query rows i    -> dQ, partial dK2/dV2   (sa2_bwd_qk2.hpp)
+//   dk2_dv2_combine   sums the partial rows -> dK2, dV2
+//   bwd_dkv1_kernel   owns rows j of K1/V1 -> dK1, dV1
 // With dlt = i - k, A = q_i * k2_{i-dlt} and B = do_i * v2_{i-dlt} (VALU, bf16):
 //   S = A K1^T, dP = B V1^T, P = exp(scale*S - lse_i), dS = P (dP - delta_i)
 //   G = dS K1 :  dq_i  += scale k2_{i-dlt} G_i     dk2_{i-dlt} += scale q_i G_i
@@ -50,7 +49,7 @@ __global__ __launch_bounds__(256) void delta_kernel(KParams p) {
     if (ok && piece == 0) p.delta[row] = s;
 }
 
-// shared pieces of the two "query-column" kernels (dQ and dK2/dV2) -----------------------
+// small GEMM helpers ---------------------------------------------------------------------
 
 // acc(32x32, rows = staged rows, column = lane column) = sum_kk lds_rows[kk] * regfrag[kk]
 template <int KS>
@@ -70,257 +69,6 @@ __device__ __forceinline__ void gemm_trans(f32x16 (&acc)[DT], const char *tbase,
         acc[dt] = mfma32(ld_lds16(b), pb[0], acc[dt]);
         acc[dt] = mfma32(ld_lds16(b + 32), pb[1], acc[dt]);
     }
-}
-
-// ------------------------------------------------------------------------------------
-// dQ: workgroup = 128 query rows of one (batch, head); same tiling as the forward.
-// ------------------------------------------------------------------------------------
-template <int D>
-__global__ __launch_bounds__(256, 1) void bwd_dq_kernel(KParams p) {
-    constexpr int KS = D / 16, DT = D / 32, CT = kChunkTiles;
-    constexpr int PK = row_pitch(D), PT = kChunkPitchT;
-    __shared__ __attribute__((aligned(16))) char k1s[kChunkRows * PK];
-    __shared__ __attribute__((aligned(16))) char v1s[kChunkRows * PK];
-    __shared__ __attribute__((aligned(16))) char k1t[D * PT];
-
-    const int N = p.N;
-    const int ntile = (N + 127) / 128;
-    const int item = xcd_contiguous(blockIdx.x, gridDim.x);
-    const int tile = ntile - 1 - item % ntile;
-    const int bh = item / ntile;
-    const int h = bh % p.H, b = bh / p.H;
-    const int hk = h / p.G;
-
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int c = lane & 31, hf = lane >> 5;
-    const int i0 = tile * 128;
-    const int iw = i0 + 32 * wave;
-    const int i = iw + c;
-    const bool row_ok = i < N;
-    const int ic = row_ok ? i : N - 1;
-
-    const char *qrow = p.q.ptr + b * p.q.sb + (int64_t)ic * p.q.sn + h * p.q.sh;
-    const char *dorow = p.dout.ptr + b * p.dout.sb + (int64_t)ic * p.dout.sn + h * p.dout.sh;
-    const char *k1g = p.k1.ptr + b * p.k1.sb + hk * p.k1.sh;
-    const char *v1g = p.v1.ptr + b * p.v1.sb + hk * p.v1.sh;
-    const char *k2g = p.k2.ptr + b * p.k2.sb + hk * p.k2.sh;
-    const char *v2g = p.v2.ptr + b * p.v2.sb + hk * p.v2.sh;
-
-    u32x4 qf[KS], dof[KS];
-#pragma unroll
-    for (int kk = 0; kk < KS; ++kk) {
-        qf[kk] = ld_global16(qrow + (16 * kk + 8 * hf) * 2);
-        dof[kk] = ld_global16(dorow + (16 * kk + 8 * hf) * 2);
-    }
-    const float lse2 = p.lse[((int64_t)b * p.H + h) * N + ic] * kLog2e;
-    const float dl = p.delta[((int64_t)b * p.H + h) * N + ic];
-
-    f32x16 dq[DT], G[DT];
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) dq[dt] = zero16();
-
-    const bool wave_active = iw < N;
-    const int wt_hi = iw / 32;
-    const int wt_lo = (iw - p.w1 + 1 > 0 ? iw - p.w1 + 1 : 0) / 32;
-    const int t_begin = (i0 - p.w1 + 1 > 0 ? i0 - p.w1 + 1 : 0) / 32;
-    const int t_end = ((i0 + 127 < N - 1) ? i0 + 127 : N - 1) / 32;
-    const int dmax = (p.w2 - 1 < iw + 31) ? p.w2 - 1 : iw + 31;
-    const float c2 = p.scale_log2e;
-    const int vrow = dmap_row(c);
-
-    for (int ct0 = t_begin; ct0 <= t_end; ct0 += CT) {
-        __syncthreads();
-        stage_rows<D>(k1s, k1g, p.k1.sn, ct0 * 32, N);
-        stage_rows<D>(v1s, v1g, p.v1.sn, ct0 * 32, N);
-        stage_rows_transposed<D>(k1t, k1g, p.k1.sn, ct0 * 32, N);
-        __syncthreads();
-        const int tl = ct0 > wt_lo ? ct0 : wt_lo;
-        const int th = (ct0 + CT - 1 < wt_hi) ? ct0 + CT - 1 : wt_hi;
-        if (!wave_active || tl > th) continue;
-
-        for (int dlt = 0; dlt <= dmax; ++dlt) {
-            const int kr = i - dlt;
-            const bool col_ok = row_ok && kr >= 0;
-            const bool any_bad = wave_any(!col_ok);
-            const int krc = kr < 0 ? 0 : (kr > N - 1 ? N - 1 : kr);
-            const char *k2row = k2g + (int64_t)krc * p.k2.sn;
-            const char *v2row = v2g + (int64_t)krc * p.v2.sn;
-            u32x4 A[KS], Bv[KS];
-#pragma unroll
-            for (int kk = 0; kk < KS; ++kk) {
-                A[kk] = mul_bf16x8(qf[kk], ld_global16(k2row + (16 * kk + 8 * hf) * 2));
-                Bv[kk] = mul_bf16x8(dof[kk], ld_global16(v2row + (16 * kk + 8 * hf) * 2));
-            }
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) G[dt] = zero16();
-
-            for (int t = tl; t <= th; ++t) {
-                const int lt = t - ct0;
-                const int roff = (32 * lt + c) * PK + 8 * hf * 2;
-                f32x16 S = gemm_rows<KS>(k1s + roff, A);
-                f32x16 dP = gemm_rows<KS>(v1s + roff, Bv);
-                const bool full = !any_bad && (t < wt_hi) && (32 * t + p.w1 > iw + 31);
-                if (!full) {
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        int j = 32 * t + 8 * (r >> 2) + 4 * hf + (r & 3);
-                        bool ok = col_ok && (j <= i) && (j + p.w1 > i);
-                        S[r] = ok ? S[r] : -INFINITY;
-                    }
-                }
-                u32x4 dsb[2];
-#pragma unroll
-                for (int r = 0; r < 16; r += 2) {
-                    float p0 = fast_exp2(S[r] * c2 - lse2);
-                    float p1 = fast_exp2(S[r + 1] * c2 - lse2);
-                    dsb[r >> 3][(r & 7) >> 1] = pack_bf16(p0 * (dP[r] - dl), p1 * (dP[r + 1] - dl));
-                }
-                gemm_trans<DT>(G, k1t + vrow * PT + (32 * lt + 8 * hf) * 2, PT, dsb);
-            }
-            fma_row<DT>(dq, G, k2row + 16 * hf * 2);
-        }
-    }
-
-    if (!row_ok) return;
-    store_row<DT>(p.dq.ptr + b * p.dq.sb + (int64_t)i * p.dq.sn + h * p.dq.sh + 16 * hf * 2, dq, p.scale);
-}
-
-// ------------------------------------------------------------------------------------
-// dK2/dV2: workgroup = 128 rows k of one (batch, kv head); lane column = k, the query
-// row met at offset dlt is i = k + dlt, so K2/V2 fragments stay in registers and the
-// q/do rows slide.  Loops over the query heads of the group.
-// ------------------------------------------------------------------------------------
-template <int D>
-__global__ __launch_bounds__(256, 1) void bwd_dkv2_kernel(KParams p) {
-    constexpr int KS = D / 16, DT = D / 32, CT = kChunkTiles;
-    constexpr int PK = row_pitch(D), PT = kChunkPitchT;
-    __shared__ __attribute__((aligned(16))) char k1s[kChunkRows * PK];
-    __shared__ __attribute__((aligned(16))) char v1s[kChunkRows * PK];
-    __shared__ __attribute__((aligned(16))) char k1t[D * PT];
-    __shared__ __attribute__((aligned(16))) char v1t[D * PT];
-
-    const int N = p.N;
-    const int ntile = (N + 127) / 128;
-    const int item = xcd_contiguous(blockIdx.x, gridDim.x);
-    const int tile = ntile - 1 - item % ntile;
-    const int bh = item / ntile;
-    const int hk = bh % p.HK, b = bh / p.HK;
-
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int c = lane & 31, hf = lane >> 5;
-    const int k0 = tile * 128;
-    const int kw = k0 + 32 * wave;
-    const int k = kw + c;
-    const bool k_ok = k < N;
-    const int kc = k_ok ? k : N - 1;
-
-    const char *k1g = p.k1.ptr + b * p.k1.sb + hk * p.k1.sh;
-    const char *v1g = p.v1.ptr + b * p.v1.sb + hk * p.v1.sh;
-    const char *k2row = p.k2.ptr + b * p.k2.sb + (int64_t)kc * p.k2.sn + hk * p.k2.sh;
-    const char *v2row = p.v2.ptr + b * p.v2.sb + (int64_t)kc * p.v2.sn + hk * p.v2.sh;
-
-    u32x4 k2f[KS], v2f[KS];
-#pragma unroll
-    for (int kk = 0; kk < KS; ++kk) {
-        k2f[kk] = ld_global16(k2row + (16 * kk + 8 * hf) * 2);
-        v2f[kk] = ld_global16(v2row + (16 * kk + 8 * hf) * 2);
-    }
-
-    f32x16 dk2[DT], dv2[DT], G[DT], T[DT];
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-        dk2[dt] = zero16();
-        dv2[dt] = zero16();
-    }
-
-    const bool wave_active = kw < N;
-    const int t_begin = (k0 - p.w1 + 1 > 0 ? k0 - p.w1 + 1 : 0) / 32;
-    const int last_i = (k0 + 127 + p.w2 - 1 < N - 1) ? k0 + 127 + p.w2 - 1 : N - 1;
-    const int t_end = last_i / 32;
-    const float c2 = p.scale_log2e;
-    const int vrow = dmap_row(c);
-
-    for (int ct0 = t_begin; ct0 <= t_end; ct0 += CT) {
-        __syncthreads();
-        stage_rows<D>(k1s, k1g, p.k1.sn, ct0 * 32, N);
-        stage_rows<D>(v1s, v1g, p.v1.sn, ct0 * 32, N);
-        stage_rows_transposed<D>(k1t, k1g, p.k1.sn, ct0 * 32, N);
-        stage_rows_transposed<D>(v1t, v1g, p.v1.sn, ct0 * 32, N);
-        __syncthreads();
-        if (!wave_active) continue;
-
-        for (int g = 0; g < p.G; ++g) {
-            const int h = hk * p.G + g;
-            const char *qg = p.q.ptr + b * p.q.sb + h * p.q.sh;
-            const char *dog = p.dout.ptr + b * p.dout.sb + h * p.dout.sh;
-            const float *lseg = p.lse + ((int64_t)b * p.H + h) * N;
-            const float *delg = p.delta + ((int64_t)b * p.H + h) * N;
-
-            for (int dlt = 0; dlt < p.w2; ++dlt) {
-                const int iw = kw + dlt;  // first query row this wave meets at this offset
-                if (iw >= N) break;
-                const int ilast = (iw + 31 < N - 1) ? iw + 31 : N - 1;
-                const int wt_hi = ilast / 32;
-                const int wt_lo = (iw - p.w1 + 1 > 0 ? iw - p.w1 + 1 : 0) / 32;
-                const int tl = ct0 > wt_lo ? ct0 : wt_lo;
-                const int th = (ct0 + CT - 1 < wt_hi) ? ct0 + CT - 1 : wt_hi;
-                if (tl > th) continue;
-
-                const int i = k + dlt;
-                const bool col_ok = k_ok && i < N;
-                const bool any_bad = wave_any(!col_ok);
-                const int ic = i < N ? i : N - 1;
-                const char *qrow = qg + (int64_t)ic * p.q.sn;
-                const char *dorow = dog + (int64_t)ic * p.dout.sn;
-                u32x4 A[KS], Bv[KS];
-#pragma unroll
-                for (int kk = 0; kk < KS; ++kk) {
-                    A[kk] = mul_bf16x8(k2f[kk], ld_global16(qrow + (16 * kk + 8 * hf) * 2));
-                    Bv[kk] = mul_bf16x8(v2f[kk], ld_global16(dorow + (16 * kk + 8 * hf) * 2));
-                }
-                const float lse2 = lseg[ic] * kLog2e;
-                const float dl = delg[ic];
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt) {
-                    G[dt] = zero16();
-                    T[dt] = zero16();
-                }
-
-                for (int t = tl; t <= th; ++t) {
-                    const int lt = t - ct0;
-                    const int roff = (32 * lt + c) * PK + 8 * hf * 2;
-                    f32x16 S = gemm_rows<KS>(k1s + roff, A);
-                    f32x16 dP = gemm_rows<KS>(v1s + roff, Bv);
-                    const bool full = !any_bad && (32 * t + 31 <= iw) && (32 * t + p.w1 > iw + 31);
-                    if (!full) {
-#pragma unroll
-                        for (int r = 0; r < 16; ++r) {
-                            int j = 32 * t + 8 * (r >> 2) + 4 * hf + (r & 3);
-                            bool ok = col_ok && (j <= i) && (j + p.w1 > i);
-                            S[r] = ok ? S[r] : -INFINITY;
-                        }
-                    }
-                    u32x4 pb[2], dsb[2];
-#pragma unroll
-                    for (int r = 0; r < 16; r += 2) {
-                        float p0 = fast_exp2(S[r] * c2 - lse2);
-                        float p1 = fast_exp2(S[r + 1] * c2 - lse2);
-                        pb[r >> 3][(r & 7) >> 1] = pack_bf16(p0, p1);
-                        dsb[r >> 3][(r & 7) >> 1] = pack_bf16(p0 * (dP[r] - dl), p1 * (dP[r + 1] - dl));
-                    }
-                    const int toff = vrow * PT + (32 * lt + 8 * hf) * 2;
-                    gemm_trans<DT>(T, v1t + toff, PT, pb);
-                    gemm_trans<DT>(G, k1t + toff, PT, dsb);
-                }
-                fma_row<DT>(dk2, G, qrow + 16 * hf * 2);
-                fma_row<DT>(dv2, T, dorow + 16 * hf * 2);
-            }
-        }
-    }
-
-    if (!k_ok) return;
-    store_row<DT>(p.dk2.ptr + b * p.dk2.sb + (int64_t)k * p.dk2.sn + hk * p.dk2.sh + 16 * hf * 2, dk2, p.scale);
-    store_row<DT>(p.dv2.ptr + b * p.dv2.sb + (int64_t)k * p.dv2.sn + hk * p.dv2.sh + 16 * hf * 2, dv2, 1.f);
 }
 
 // ------------------------------------------------------------------------------------

@@ -70,6 +70,12 @@ __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(a), as_bf16x8(b), c, 0, 0, 0);
 }
 
+// Keeps an MFMA accumulator in accumulation registers at this point of the program.
+// VALU instructions cannot read those registers, so without the pin the compiler may
+// decide to hold a rarely VALU-touched accumulator in ordinary registers for a whole
+// loop and copy all of it to and from the MFMA's registers on every iteration.
+__device__ __forceinline__ void pin_acc(f32x16 &x) { asm volatile("" : "+a"(x)); }
+
 __device__ __forceinline__ f32x16 zero16() {
     f32x16 z;
 #pragma unroll

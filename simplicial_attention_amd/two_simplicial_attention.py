@@ -59,7 +59,7 @@ class SlidingTwoSimplicialAttention(Function):
             raise ValueError('window sizes must be at least 1')
         lib = _native.load()
         if not lib.sa2_supported(dim, w1, w2, _native.SA2_BF16):
-            raise NotImplementedError(f'dim_head={dim}, w1={w1}, w2={w2} is not covered by the kernels (dim_head 64 or 128)')
+            raise NotImplementedError(f'dim_head={dim}, w1={w1}, w2={w2} is not covered by the kernels (dim_head 64 or 128, w2 <= 64)')
 
         q, k1, k2, v1, v2 = (_unit_inner_stride(t) for t in tensors)
         scale = dim ** -0.5
@@ -87,12 +87,15 @@ class SlidingTwoSimplicialAttention(Function):
         dq = torch.empty_like(q)
         dk1, dk2, dv1, dv2 = (torch.empty((batch, seq_len, kv_heads, dim), dtype=q.dtype, device=q.device) for _ in range(4))
         prob = _native.problem(batch, seq_len, heads, kv_heads, dim, w1, w2, True, scale)
+        ws_bytes = lib.sa2_bwd_workspace_bytes(prob)
+        workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
         arg = _native.tensor_arg
         with torch.cuda.device_of(q):
             _native.check(lib.sa2_bwd(prob, arg(q), arg(k1), arg(k2), arg(v1), arg(v2), arg(out),
                                       arg(residual) if residual is not None else None, arg(dout),
                                       lse.data_ptr(), delta.data_ptr(),
-                                      arg(dq), arg(dk1), arg(dk2), arg(dv1), arg(dv2), _stream_handle(q.device)))
+                                      arg(dq), arg(dk1), arg(dk2), arg(dv1), arg(dv2),
+                                      workspace.data_ptr(), ws_bytes, _stream_handle(q.device)))
         return dq, dk1, dk2, dv1, dv2, None, None, None
 
 

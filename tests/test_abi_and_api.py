@@ -39,6 +39,7 @@ def test_every_declared_symbol_is_exported(lib):
 def test_supported_matrix(lib):
     assert lib.sa2_supported(64, 512, 32, 0) == 1
     assert lib.sa2_supported(128, 512, 64, 0) == 1
+    assert lib.sa2_supported(128, 512, 65, 0) == 0
     assert lib.sa2_supported(32, 512, 32, 0) == 0
     assert lib.sa2_supported(128, 0, 32, 0) == 0
     assert lib.sa2_supported(128, 512, 32, 1) == 0
@@ -73,10 +74,15 @@ def test_argument_validation_happens_before_any_launch(lib):
     assert 'SA2_ERR_ALIGNMENT' in str(e.value) and 'k2' in str(e.value)
     # backward entry points validate the same way
     assert lib.sa2_bwd_delta(good, None, None, t, lse, None) == 1
-    assert lib.sa2_bwd_dq(good, t, t, t, t, t, t, None, lse, t, None) == 1
+    need = lib.sa2_bwd_workspace_bytes(good)
+    assert need == 2 * 1 * 2 * 2 * 63 * 128 * 4          # 2 tensors, B*H*tiles blocks of 63 fp32 rows
+    assert lib.sa2_bwd_workspace_bytes(None) == -1
+    assert lib.sa2_bwd_dq_dkv2(good, t, t, t, t, t, t, None, lse, t, t, t, lse, need, None) == 1
+    assert lib.sa2_bwd_dq_dkv2(good, t, t, t, t, t, t, lse, lse, t, t, t, None, need, None) == 1
+    assert lib.sa2_bwd_dq_dkv2(good, t, t, t, t, t, t, lse, lse, t, t, t, lse, need - 1, None) == 2
+    assert lib.sa2_bwd_dq_dkv2(good, t, t, t, t, t, t, lse, lse, t, t, _dummy(ptr=0x1004), lse, need, None) == 4
     assert lib.sa2_bwd_dkv1(good, t, t, t, t, t, t, lse, lse, None, t, None) == 1
-    assert lib.sa2_bwd_dkv2(good, t, t, t, t, t, t, lse, lse, t, _dummy(ptr=0x1004), None) == 4
-    assert lib.sa2_bwd(good, t, t, t, t, t, None, None, t, lse, lse, t, t, t, t, t, None) == 1
+    assert lib.sa2_bwd(good, t, t, t, t, t, None, None, t, lse, lse, t, t, t, t, t, lse, need, None) == 1
 
 
 def test_function_rejects_what_the_kernels_do_not_cover():
