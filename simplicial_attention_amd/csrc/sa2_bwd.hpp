@@ -16,6 +16,7 @@
 #pragma once
 
 #include "sa2_common.hpp"
+#include "sa2_fwd_ds.hpp"
 
 namespace sa2 {
 
@@ -72,28 +73,30 @@ __device__ __forceinline__ void gemm_trans(f32x16 (&acc)[DT], const char *tbase,
 }
 
 // ------------------------------------------------------------------------------------
-// dK1/dV1: workgroup = 128 rows j of one (batch, kv head); lane column = j, K1/V1
-// fragments stay in registers as B operands.  For every (32-row query tile, offset dlt)
-// the workgroup builds A = q*k2 and B = do*v2 once in LDS, row-major (operands of S
-// and dP) and transposed (operands of dV1^T += B^T P and dK1^T += A^T dS).
+// dK1/dV1: workgroup = 128 rows j of one (batch, kv head); wave w owns rows
+// [32w, 32w+32), lane column = j, and keeps its K1/V1 fragments in registers as B
+// operands.  The workgroup walks "steps" = (query head of the group, 32-row query
+// tile, offset dlt).  For every step the 256 threads build A = q*k2 and B = do*v2
+// (32 x D each) once, row-major in LDS; the row-major fragments feed S and dP, and
+// ds_read_b64_tr_b16 reads of the same tiles feed dV1^T += B^T P and dK1^T += A^T dS.
+// Tiles are double buffered: the products of step s+1 are written while step s
+// computes, their global loads are issued one step earlier still.
 // ------------------------------------------------------------------------------------
 template <int D>
-struct Dkv1Buf {
-    static constexpr int PK = row_pitch(D);
-    static constexpr int PT = (32 + 8) * 2;
-    static constexpr int AS = 0;
-    static constexpr int BS = AS + 32 * PK;
-    static constexpr int AT = BS + 32 * PK;
-    static constexpr int BT = AT + D * PT;
-    static constexpr int LSE = BT + D * PT;
-    static constexpr int DEL = LSE + 32 * 4;
+struct Dkv1Cfg {
+    static constexpr int TILE = 32 * tile_pitch<D>();
+    static constexpr int AS = 0;                 // A tile
+    static constexpr int BS = TILE;              // B tile
+    static constexpr int LSE = 2 * TILE;         // 32 floats: lse * log2e (+inf for dead rows)
+    static constexpr int DEL = LSE + 32 * 4;     // 32 floats: delta
     static constexpr int BYTES = DEL + 32 * 4;
+    static constexpr int LPT = 32 * D / 8 / 256; // 16-byte pieces per thread and tensor
 };
 
 template <int D>
-__global__ __launch_bounds__(256, 2) void bwd_dkv1_kernel(KParams p) {
-    constexpr int KS = D / 16, DT = D / 32;
-    using L = Dkv1Buf<D>;
+__global__ __launch_bounds__(256, 1) void bwd_dkv1_kernel(KParams p) {
+    constexpr int KS = D / 16, DT = D / 32, PPR = D / 8, PITCH = tile_pitch<D>();
+    using L = Dkv1Cfg<D>;
     __shared__ __attribute__((aligned(16))) char lds[2 * L::BYTES];
 
     const int N = p.N;
@@ -137,90 +140,144 @@ __global__ __launch_bounds__(256, 2) void bwd_dkv1_kernel(KParams p) {
     const int wit_lo = jw / 32;
     const int wit_hi = ((jw + 31 + p.w1 - 1 < N - 1) ? jw + 31 + p.w1 - 1 : N - 1) / 32;
     const float c2 = p.scale_log2e;
-    const int vrow = dmap_row(c);
-    constexpr int PPR = D / 8;
+    const int r_lane = c * PITCH + 16 * hf;
+    const int t_lane = tr_lane_off<D>(lane);
 
-    int step = 0;
-    for (int g = 0; g < p.G; ++g) {
-        const int h = hk * p.G + g;
-        const char *qg = p.q.ptr + b * p.q.sb + h * p.q.sh;
-        const char *dog = p.dout.ptr + b * p.dout.sb + h * p.dout.sh;
-        const float *lseg = p.lse + ((int64_t)b * p.H + h) * N;
-        const float *delg = p.delta + ((int64_t)b * p.H + h) * N;
-
-        for (int it = it_begin; it <= it_end; ++it) {
-            const int dmax = (p.w2 - 1 < 32 * it + 31) ? p.w2 - 1 : 32 * it + 31;
-            for (int dlt = 0; dlt <= dmax; ++dlt, ++step) {
-                char *buf = lds + (step & 1) * L::BYTES;
-                // ---- build A, B (row-major and transposed), lse, delta for this step
-#pragma unroll
-                for (int rep = 0; rep < 32 * PPR / 256; ++rep) {
-                    const int idx = rep * 256 + tid;
-                    const int il = idx / PPR, piece = idx % PPR;
-                    const int i = 32 * it + il;
-                    const int kr = i - dlt;
-                    const bool valid = i < N && kr >= 0;
-                    u32x4 a = {0u, 0u, 0u, 0u}, bb = {0u, 0u, 0u, 0u};
-                    if (valid) {
-                        a = mul_bf16x8(ld_global16(qg + (int64_t)i * p.q.sn + piece * 16),
-                                       ld_global16(k2g + (int64_t)kr * p.k2.sn + piece * 16));
-                        bb = mul_bf16x8(ld_global16(dog + (int64_t)i * p.dout.sn + piece * 16),
-                                        ld_global16(v2g + (int64_t)kr * p.v2.sn + piece * 16));
-                    }
-                    *reinterpret_cast<u32x4 *>(buf + L::AS + il * L::PK + piece * 16) = a;
-                    *reinterpret_cast<u32x4 *>(buf + L::BS + il * L::PK + piece * 16) = bb;
-                    const int pos = kslot_pos(il);
-#pragma unroll
-                    for (int w = 0; w < 4; ++w) {
-                        const int d = 8 * piece + 2 * w;
-                        *reinterpret_cast<uint16_t *>(buf + L::AT + d * L::PT + pos * 2) = (uint16_t)(a[w] & 0xffffu);
-                        *reinterpret_cast<uint16_t *>(buf + L::AT + (d + 1) * L::PT + pos * 2) = (uint16_t)(a[w] >> 16);
-                        *reinterpret_cast<uint16_t *>(buf + L::BT + d * L::PT + pos * 2) = (uint16_t)(bb[w] & 0xffffu);
-                        *reinterpret_cast<uint16_t *>(buf + L::BT + (d + 1) * L::PT + pos * 2) = (uint16_t)(bb[w] >> 16);
-                    }
-                }
-                if (tid < 32) {
-                    const int i = 32 * it + tid;
-                    const bool valid = i < N && i - dlt >= 0;
-                    reinterpret_cast<float *>(buf + L::LSE)[tid] = valid ? lseg[i] * kLog2e : INFINITY;
-                    reinterpret_cast<float *>(buf + L::DEL)[tid] = valid ? delg[i] : 0.f;
-                }
-                __syncthreads();
-                if (!wave_active || it < wit_lo || it > wit_hi) continue;
-
-                // ---- S[i,j], dP[i,j]: rows = query rows of the tile, column = j
-                const int roff = c * L::PK + 8 * hf * 2;
-                f32x16 S = gemm_rows<KS>(buf + L::AS + roff, k1f);
-                f32x16 dP = gemm_rows<KS>(buf + L::BS + roff, v1f);
-                const bool full = (jw + 31 <= 32 * it) && (jw + p.w1 > 32 * it + 31);
-                if (!full) {
-#pragma unroll
-                    for (int r = 0; r < 16; ++r) {
-                        int i = 32 * it + 8 * (r >> 2) + 4 * hf + (r & 3);
-                        bool ok = (j <= i) && (j + p.w1 > i);
-                        S[r] = ok ? S[r] : -INFINITY;
-                    }
-                }
-                u32x4 pb[2], dsb[2];
-#pragma unroll
-                for (int a4 = 0; a4 < 4; ++a4) {
-                    const float4 l4 = *reinterpret_cast<const float4 *>(buf + L::LSE + (8 * a4 + 4 * hf) * 4);
-                    const float4 d4 = *reinterpret_cast<const float4 *>(buf + L::DEL + (8 * a4 + 4 * hf) * 4);
-                    const int r = 4 * a4;
-                    float p0 = fast_exp2(S[r] * c2 - l4.x);
-                    float p1 = fast_exp2(S[r + 1] * c2 - l4.y);
-                    float p2 = fast_exp2(S[r + 2] * c2 - l4.z);
-                    float p3 = fast_exp2(S[r + 3] * c2 - l4.w);
-                    pb[a4 >> 1][2 * (a4 & 1)] = pack_bf16(p0, p1);
-                    pb[a4 >> 1][2 * (a4 & 1) + 1] = pack_bf16(p2, p3);
-                    dsb[a4 >> 1][2 * (a4 & 1)] = pack_bf16(p0 * (dP[r] - d4.x), p1 * (dP[r + 1] - d4.y));
-                    dsb[a4 >> 1][2 * (a4 & 1) + 1] = pack_bf16(p2 * (dP[r + 2] - d4.z), p3 * (dP[r + 3] - d4.w));
-                }
-                const int toff = vrow * L::PT + 8 * hf * 2;
-                gemm_trans<DT>(dv1, buf + L::BT + toff, L::PT, pb);
-                gemm_trans<DT>(dk1, buf + L::AT + toff, L::PT, dsb);
+    // ---- step iterator (g, it, dlt) for the loads, which run two steps ahead
+    struct Step {
+        int g, it, dlt;
+    };
+    auto dmax_of = [&](int it) { return (p.w2 - 1 < 32 * it + 31) ? p.w2 - 1 : 32 * it + 31; };
+    auto next_step = [&](Step &s) {
+        if (++s.dlt > dmax_of(s.it)) {
+            s.dlt = 0;
+            if (++s.it > it_end) {
+                s.it = it_begin;
+                ++s.g;
             }
         }
+    };
+    int nsteps = 0;
+    for (int it = it_begin; it <= it_end; ++it) nsteps += dmax_of(it) + 1;
+    nsteps *= p.G;
+
+    // ---- operand staging: each thread owns LPT 16-byte pieces of the A and of the B tile
+    u32x4 lq[L::LPT], lk[L::LPT], lo[L::LPT], lv[L::LPT];
+    float l_lse = 0.f, l_del = 0.f;
+    int st_off[L::LPT];
+#pragma unroll
+    for (int x = 0; x < L::LPT; ++x) st_off[x] = ((x * 256 + tid) / PPR) * PITCH + ((x * 256 + tid) % PPR) * 16;
+    auto issue_loads = [&](const Step &s) {
+        const int h = hk * p.G + s.g;
+        const char *qg = p.q.ptr + b * p.q.sb + h * p.q.sh;
+        const char *dog = p.dout.ptr + b * p.dout.sb + h * p.dout.sh;
+#pragma unroll
+        for (int x = 0; x < L::LPT; ++x) {
+            const int pc = x * 256 + tid;
+            int i = 32 * s.it + pc / PPR;
+            int kr = i - s.dlt;
+            i = i < N ? i : N - 1;
+            kr = kr < 0 ? 0 : (kr < N ? kr : N - 1);
+            const int col = (pc % PPR) * 16;
+            lq[x] = ld_global16(qg + (int64_t)i * p.q.sn + col);
+            lk[x] = ld_global16(k2g + (int64_t)kr * p.k2.sn + col);
+            lo[x] = ld_global16(dog + (int64_t)i * p.dout.sn + col);
+            lv[x] = ld_global16(v2g + (int64_t)kr * p.v2.sn + col);
+        }
+        if (tid < 32) {
+            const int i = 32 * s.it + tid;
+            const bool valid = i < N && i - s.dlt >= 0;
+            const int icl = i < N ? i : N - 1;
+            l_lse = valid ? p.lse[((int64_t)b * p.H + h) * N + icl] * kLog2e : INFINITY;
+            l_del = valid ? p.delta[((int64_t)b * p.H + h) * N + icl] : 0.f;
+        }
+    };
+    auto write_stage = [&](int buf) {
+        char *stage = lds + buf * L::BYTES;
+#pragma unroll
+        for (int x = 0; x < L::LPT; ++x) {
+            *reinterpret_cast<u32x4 *>(stage + L::AS + st_off[x]) = mul_bf16x8(lq[x], lk[x]);
+            *reinterpret_cast<u32x4 *>(stage + L::BS + st_off[x]) = mul_bf16x8(lo[x], lv[x]);
+        }
+        if (tid < 32) {
+            reinterpret_cast<float *>(stage + L::LSE)[tid] = l_lse;
+            reinterpret_cast<float *>(stage + L::DEL)[tid] = l_del;
+        }
+    };
+
+    Step ld = {0, it_begin, 0};   // next step to load
+    Step cur = {0, it_begin, 0};  // step being computed
+    issue_loads(ld);
+    next_step(ld);
+    write_stage(0);
+    if (nsteps > 1) {
+        issue_loads(ld);
+        next_step(ld);
+    }
+
+    for (int s = 0; s < nsteps; ++s) {
+        __syncthreads();
+        if (s + 1 < nsteps) write_stage((s + 1) & 1);
+        if (s + 2 < nsteps) {
+            issue_loads(ld);
+            next_step(ld);
+        }
+        const char *buf = lds + (s & 1) * L::BYTES;
+        const int it = cur.it;
+        next_step(cur);
+        if (!wave_active || it < wit_lo || it > wit_hi) continue;
+
+        // ---- S[i,j], dP[i,j]: rows = query rows of the tile, column = j
+        f32x16 X = zero16(), dP = zero16();
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk) {
+            X = mfma32(ld_lds16(buf + L::AS + r_lane + 32 * kk), k1f[kk], X);
+            dP = mfma32(ld_lds16(buf + L::BS + r_lane + 32 * kk), v1f[kk], dP);
+        }
+        float dls[16];
+#pragma unroll
+        for (int a4 = 0; a4 < 4; ++a4) {
+            const float4 l4 = *reinterpret_cast<const float4 *>(buf + L::LSE + (8 * a4 + 4 * hf) * 4);
+            const float4 d4 = *reinterpret_cast<const float4 *>(buf + L::DEL + (8 * a4 + 4 * hf) * 4);
+            X[4 * a4] = X[4 * a4] * c2 - l4.x;
+            X[4 * a4 + 1] = X[4 * a4 + 1] * c2 - l4.y;
+            X[4 * a4 + 2] = X[4 * a4 + 2] * c2 - l4.z;
+            X[4 * a4 + 3] = X[4 * a4 + 3] * c2 - l4.w;
+            dls[4 * a4] = d4.x;
+            dls[4 * a4 + 1] = d4.y;
+            dls[4 * a4 + 2] = d4.z;
+            dls[4 * a4 + 3] = d4.w;
+        }
+        const bool full = (jw + 31 <= 32 * it) && (jw + p.w1 > 32 * it + 31);
+        if (!full) {
+            const int base = 32 * it + 4 * hf - j;   // i - j for register 0
+#pragma unroll
+            for (int rr = 0; rr < 16; ++rr) {
+                const bool ok = (unsigned)(base + 8 * (rr >> 2) + (rr & 3)) < (unsigned)p.w1;
+                X[rr] = ok ? X[rr] : -INFINITY;
+            }
+        }
+        u32x4 pb[2], dsb[2];
+#pragma unroll
+        for (int rr = 0; rr < 16; rr += 2) {
+            float p0 = fast_exp2(X[rr]);
+            float p1 = fast_exp2(X[rr + 1]);
+            pb[rr >> 3][(rr & 7) >> 1] = pack_bf16(p0, p1);
+            dsb[rr >> 3][(rr & 7) >> 1] = pack_bf16(p0 * (dP[rr] - dls[rr]), p1 * (dP[rr + 1] - dls[rr + 1]));
+        }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int k2s = 0; k2s < 2; ++k2s) {
+                u32x2 blo = lds_read_tr<D>(buf + L::BS + t_lane, 16 * k2s, 32 * dt);
+                u32x2 bhi = lds_read_tr<D>(buf + L::BS + t_lane, 16 * k2s + 8, 32 * dt);
+                u32x2 alo = lds_read_tr<D>(buf + L::AS + t_lane, 16 * k2s, 32 * dt);
+                u32x2 ahi = lds_read_tr<D>(buf + L::AS + t_lane, 16 * k2s + 8, 32 * dt);
+                u32x4 bfr = {blo[0], blo[1], bhi[0], bhi[1]};
+                u32x4 afr = {alo[0], alo[1], ahi[0], ahi[1]};
+                dv1[dt] = mfma32(bfr, pb[k2s], dv1[dt]);
+                dk1[dt] = mfma32(afr, dsb[k2s], dk1[dt]);
+            }
     }
 
     if (!j_ok) return;
