@@ -131,6 +131,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv1_kernel(KParams p) {
     for (int dt = 0; dt < DT; ++dt) {
         dk1[dt] = zero16();
         dv1[dt] = zero16();
+        pin_acc(dk1[dt]);
+        pin_acc(dv1[dt]);
     }
 
     const int it_begin = j0 / 32;
@@ -278,6 +280,11 @@ __global__ __launch_bounds__(256, 1) void bwd_dkv1_kernel(KParams p) {
                 dv1[dt] = mfma32(bfr, pb[k2s], dv1[dt]);
                 dk1[dt] = mfma32(afr, dsb[k2s], dk1[dt]);
             }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) {
+            pin_acc(dk1[dt]);
+            pin_acc(dv1[dt]);
+        }
     }
 
     if (!j_ok) return;

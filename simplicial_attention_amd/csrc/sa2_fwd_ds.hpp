@@ -19,6 +19,10 @@
 
 #include "sa2_common.hpp"
 
+#ifndef SA2_SCHED
+#define SA2_SCHED 1
+#endif
+
 namespace sa2 {
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -52,7 +56,7 @@ struct FwdDs {
     static constexpr int KS = D / 16;
     static constexpr int DT = D / 32;
     static constexpr int TILE = 32 * tile_pitch<D>();  // bytes of one padded [32][D] bf16 tile
-    static constexpr int NBUF = 3;
+    static constexpr int NBUF = 4;
     static constexpr int STAGE = 2 * TILE;            // K1 tile + V1 tile
     static constexpr int RING = NBUF * STAGE;
     static constexpr int APITCH = D + 4;              // floats per row of a parked accumulator
@@ -146,20 +150,36 @@ __global__ __launch_bounds__(256, 1) void fwd_ds_kernel(KParams p) {
     float seen = -INFINITY;   // running maximum of x relative to M; -inf: no valid entry yet
     float l = 0.f, acc_scale = 1.f;
 
-    // ring bookkeeping: tile index of the next load / next stage to fill / stage in use
-    int t_load = t_lo, buf_fill = 0, buf_use = 0, u_load = 0;
-    auto advance_load = [&]() {
-        ++u_load;
-        t_load = (t_load == t_hi) ? t_lo : t_load + 1;
-    };
-    issue_loads(t_load);
-    advance_load();
-    write_stage(0);
-    buf_fill = 1;
-    if (U > 1) {
+    // ---- LDS ring of NBUF = 4 stages, indexed by the running tile counter u (tiles of
+    // successive rounds follow each other).  Invariant at the top of the step that
+    // consumes tile u: tiles u .. u+2 are in LDS, the data of tile u+3 sits in the
+    // staging registers, the K1 fragments of tile u+1 are already in registers.
+    int t_load = t_lo;                       // tile index (within the window) of the next global load
+    auto advance_load = [&]() { t_load = (t_load == t_hi) ? t_lo : t_load + 1; };
+    int buf_fill = 0, buf_use = 0;
+    auto next_buf = [&](int b) { return b == C::NBUF - 1 ? 0 : b + 1; };
+#pragma unroll
+    for (int x = 0; x < 3; ++x) {
         issue_loads(t_load);
         advance_load();
+        write_stage(buf_fill);
+        buf_fill = next_buf(buf_fill);
     }
+    issue_loads(t_load);
+    advance_load();
+    __syncthreads();
+
+    u32x4 kf[KS];                            // K1 fragments of the tile whose logits are computed next
+    auto load_kf = [&](int buf) {
+        const char *kbase = lds + buf * C::STAGE + k_lane;
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk) kf[kk] = ld_lds16(kbase + 32 * kk);
+    };
+    load_kf(0);
+    int buf_k = 1;                           // stage holding the tile after the one in kf
+
+    f32x16 Xc[2];                            // processed logits (relative to M, log2 domain) of the current tile
+    float tmax = 0.f;
 
     for (int r = 0; r < R; ++r) {
         bool col_ok[2], any_bad[2];
@@ -179,131 +199,178 @@ __global__ __launch_bounds__(256, 1) void fwd_ds_kernel(KParams p) {
             for (int dt = 0; dt < DT; ++dt) T[s][dt] = zero16();
         }
 
-        f32x16 X[2];          // logits of the current tile relative to M (log2 domain)
-        float tmax = 0.f;
-        u32x2 vf[DT][2][2];   // V1 fragments of the current tile (prefetched with the K1 ones)
-        // exponentials, row sums and T^T += V1^T P^T for the tile whose logits are in X
-        auto finish_tile = [&]() {
+        float lp[4] = {0.f, 0.f, 0.f, 0.f};     // partial row sums of this round
+        // logits of a tile from the fragments in kf: every fragment feeds both streams
+        auto s_gemm = [&](f32x16 (&X)[2]) {
+            X[0] = zero16();
+            X[1] = zero16();
 #pragma unroll
-            for (int s = 0; s < 2; ++s) {
-                u32x4 pb[2];
-#pragma unroll
-                for (int rr = 0; rr < 16; rr += 2) {
-                    float p0 = fast_exp2(X[s][rr]);
-                    float p1 = fast_exp2(X[s][rr + 1]);
-                    l += p0 + p1;
-                    pb[rr >> 3][(rr & 7) >> 1] = pack_bf16(p0, p1);
-                }
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                    for (int k2s = 0; k2s < 2; ++k2s) {
-                        u32x4 v = {vf[dt][k2s][0][0], vf[dt][k2s][0][1], vf[dt][k2s][1][0], vf[dt][k2s][1][1]};
-                        T[s][dt] = mfma32(v, pb[k2s], T[s][dt]);
-                    }
+            for (int kk = 0; kk < KS; ++kk) {
+                X[0] = mfma32(kf[kk], A[0][kk], X[0]);
+                X[1] = mfma32(kf[kk], A[1][kk], X[1]);
             }
         };
-        // One pass over tiles [t, t_end]; MASKED selects the boundary-tile code.  Returns
-        // true if it stopped at tile t because some row left the safe exponent range
-        // (X, tmax and the fragments of that tile are then still live).
-        auto run_tiles = [&](int &t, int t_end, auto masked_tag) -> bool {
+        // raw logits of tile t -> Xc (scaled, referenced, masked) and their row maximum
+        auto post_s = [&](const f32x16 (&X)[2], int t, auto masked_tag) {
             constexpr bool MASKED = decltype(masked_tag)::value;
-            for (; t <= t_end; ++t) {
-                __syncthreads();
-                // the stage written before this barrier is visible; refill the ring behind it
-                if (u_load - 1 > r * NT + (t - t_lo)) {
-                    write_stage(buf_fill);
-                    buf_fill = buf_fill == C::NBUF - 1 ? 0 : buf_fill + 1;
-                }
-                if (u_load < U) {
-                    issue_loads(t_load);
-                    advance_load();
-                }
-                const char *kbase = lds + buf_use * C::STAGE + k_lane;
-                const char *vbase = lds + buf_use * C::STAGE + v_lane;
-                buf_use = buf_use == C::NBUF - 1 ? 0 : buf_use + 1;
-
-                // ---- operand fragments of this tile, all issued up front
-                u32x4 kf[KS];
 #pragma unroll
-                for (int kk = 0; kk < KS; ++kk) kf[kk] = ld_lds16(kbase + 32 * kk);
+            for (int s = 0; s < 2; ++s)
 #pragma unroll
-                for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                    for (int k2s = 0; k2s < 2; ++k2s) {
-                        vf[dt][k2s][0] = lds_read_tr<D>(vbase, 16 * k2s, 32 * dt);
-                        vf[dt][k2s][1] = lds_read_tr<D>(vbase, 16 * k2s + 8, 32 * dt);
-                    }
-                // ---- logits of both streams; every K1 fragment feeds two MFMAs
-                X[0] = zero16();
-                X[1] = zero16();
-#pragma unroll
-                for (int kk = 0; kk < KS; ++kk) {
-                    X[0] = mfma32(kf[kk], A[0][kk], X[0]);
-                    X[1] = mfma32(kf[kk], A[1][kk], X[1]);
-                }
+                for (int rr = 0; rr < 16; ++rr) Xc[s][rr] = X[s][rr] * c2 - M;
+            if constexpr (MASKED) {
 #pragma unroll
                 for (int s = 0; s < 2; ++s)
 #pragma unroll
-                    for (int rr = 0; rr < 16; ++rr) X[s][rr] = X[s][rr] * c2 - M;
-                if constexpr (MASKED) {
+                    for (int rr = 0; rr < 16; ++rr) {
+                        int j = 32 * t + 8 * (rr >> 2) + 4 * hf + (rr & 3);
+                        bool ok = col_ok[s] && (j <= i) && (j + p.w1 > i);
+                        Xc[s][rr] = ok ? Xc[s][rr] : -INFINITY;
+                    }
+            }
+            tmax = fmaxf(Xc[0][0], Xc[1][0]);
 #pragma unroll
-                    for (int s = 0; s < 2; ++s)
+            for (int rr = 1; rr < 16; ++rr) tmax = fmaxf(tmax, fmaxf(Xc[0][rr], Xc[1][rr]));
+            auto sw = __builtin_amdgcn_permlane32_swap(as_u32(tmax), as_u32(tmax), false, false);
+            tmax = fmaxf(as_f32(sw[0]), as_f32(sw[1]));
+        };
+        // x must stay inside the safe exponent range.  The rare slow path moves the reference
+        // of the rows that left it and rescales what the accumulators already hold; it is
+        // kept OUT of the pipelined loop (the loop returns to it), because VALU code that
+        // touches T inside the loop makes the compiler copy T out of the accumulation
+        // registers on every iteration.
+        auto out_of_range = [&]() {
+            return wave_any(tmax > 64.f || (seen == -INFINITY && tmax < -32.f && tmax > -INFINITY));
+        };
+        auto slow_path = [&]() {
+            const bool fresh = seen == -INFINITY;
+            const bool move = tmax > 64.f || (fresh && tmax < -32.f && tmax > -INFINITY);
+            const float shift = move ? tmax : 0.f;
+            const float alpha = fresh ? 1.f : fast_exp2(-shift);   // fresh rows hold T = l = 0
 #pragma unroll
-                        for (int rr = 0; rr < 16; ++rr) {
-                            int j = 32 * t + 8 * (rr >> 2) + 4 * hf + (rr & 3);
-                            bool ok = col_ok[s] && (j <= i) && (j + p.w1 > i);
-                            X[s][rr] = ok ? X[s][rr] : -INFINITY;
-                        }
+            for (int s = 0; s < 2; ++s) {
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int rr = 0; rr < 16; ++rr) T[s][dt][rr] *= alpha;
+#pragma unroll
+                for (int rr = 0; rr < 16; ++rr) Xc[s][rr] -= shift;
+            }
+            l *= alpha;
+#pragma unroll
+            for (int x = 0; x < 4; ++x) lp[x] *= alpha;
+            acc_scale *= alpha;
+            M += shift;
+            seen = fmaxf(seen - shift, tmax - shift);
+        };
+        // exponentials of the current tile -> packed bf16 B operands, row sums into l
+        u32x4 pb[2][2];
+        auto exps = [&]() {
+#pragma unroll
+            for (int s = 0; s < 2; ++s)
+#pragma unroll
+                for (int rr = 0; rr < 16; rr += 2) {
+                    float p0 = fast_exp2(Xc[s][rr]);
+                    float p1 = fast_exp2(Xc[s][rr + 1]);
+                    lp[(rr >> 1) & 3] += p0 + p1;
+                    pb[s][rr >> 3][(rr & 7) >> 1] = pack_bf16(p0, p1);
                 }
-                tmax = fmaxf(X[0][0], X[1][0]);
+        };
+        u32x2 vf[DT][2][2];
+        auto load_vf = [&](int buf) {
+            const char *vbase = lds + buf * C::STAGE + v_lane;
 #pragma unroll
-                for (int rr = 1; rr < 16; ++rr) tmax = fmaxf(tmax, fmaxf(X[0][rr], X[1][rr]));
-                {
-                    auto sw = __builtin_amdgcn_permlane32_swap(as_u32(tmax), as_u32(tmax), false, false);
-                    tmax = fmaxf(as_f32(sw[0]), as_f32(sw[1]));
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int k2s = 0; k2s < 2; ++k2s) {
+                    vf[dt][k2s][0] = lds_read_tr<D>(vbase, 16 * k2s, 32 * dt);
+                    vf[dt][k2s][1] = lds_read_tr<D>(vbase, 16 * k2s + 8, 32 * dt);
                 }
-                if (wave_any(tmax > 64.f || (seen == -INFINITY && tmax < -32.f && tmax > -INFINITY))) return true;
+        };
+        auto t_gemm = [&]() {
+#pragma unroll
+            for (int k2s = 0; k2s < 2; ++k2s)
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    u32x4 v = {vf[dt][k2s][0][0], vf[dt][k2s][0][1], vf[dt][k2s][1][0], vf[dt][k2s][1][1]};
+                    T[0][dt] = mfma32(v, pb[0][k2s], T[0][dt]);
+                    T[1][dt] = mfma32(v, pb[1][k2s], T[1][dt]);
+                }
+        };
+        // barrier + refill of the ring: stage u+3 is written, the loads of tile u+4 issued
+        auto sync_and_refill = [&]() {
+            __syncthreads();
+            write_stage(buf_fill);
+            buf_fill = next_buf(buf_fill);
+            issue_loads(t_load);
+            advance_load();
+        };
+
+        // ---- round prologue: logits of the first tile (its K1 fragments are in kf)
+        {
+            f32x16 Xn[2];
+            s_gemm(Xn);
+            load_kf(buf_k);
+            buf_k = next_buf(buf_k);
+            post_s(Xn, t_lo, std::true_type{});
+            if (out_of_range()) slow_path();
+            else seen = fmaxf(seen, tmax);
+        }
+        // ---- pipelined steps: exponentials and T-GEMM of tile t overlap with the logit
+        // GEMM and the logit post-processing of tile t+1
+        int mid_lo = (i0 + 31 - p.w1 >= 0) ? (i0 + 31 - p.w1) / 32 + 1 : t_lo;
+        if (any_bad[0] || any_bad[1]) mid_lo = t_hi;
+        mid_lo = mid_lo > t_hi ? t_hi : mid_lo;
+        // runs steps t .. t_end; returns true if it stopped early (t already advanced)
+        // because the logits just produced left the safe range
+        auto steps = [&](int &t, int t_end, auto masked_tag) -> bool {
+            while (t <= t_end) {                 // consumes tile t, produces the logits of tile t+1
+                sync_and_refill();
+                load_vf(buf_use);
+                buf_use = next_buf(buf_use);
+                f32x16 Xn[2];
+                s_gemm(Xn);
+                exps();
+                load_kf(buf_k);
+                buf_k = next_buf(buf_k);
+                t_gemm();
+                post_s(Xn, t + 1, masked_tag);
+#if SA2_SCHED
+                // phase 1: 16 logit MFMAs, each followed by a share of the exponential work
+                // and one of the 16 transposed V1 fragment reads
+#pragma unroll
+                for (int x = 0; x < 16; ++x) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, 5, 0);
+                }
+                // phase 2: 16 value MFMAs, each followed by a share of the post-processing
+                // of the next logits; the first 8 also by one K1 fragment read
+#pragma unroll
+                for (int x = 0; x < 16; ++x) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    if (x < 8) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, 6, 0);
+                }
+#endif
+                ++t;
+                if (out_of_range()) return true;
                 seen = fmaxf(seen, tmax);
-                finish_tile();
             }
             return false;
         };
-
-        // tiles [t_lo, t_hi] = masked head | unmasked middle | masked tail (the diagonal)
-        int mid_lo = (i0 + 31 - p.w1 >= 0) ? (i0 + 31 - p.w1) / 32 + 1 : t_lo;
-        if (any_bad[0] || any_bad[1]) mid_lo = t_hi + 1;      // edge rows: mask everywhere
-        mid_lo = mid_lo > t_hi ? t_hi : mid_lo;               // the diagonal tile is always masked
-        const int seg_end[3] = {mid_lo - 1, t_hi - 1, t_hi};
-        int t = t_lo;
-#pragma unroll
-        for (int seg = 0; seg < 3; ++seg) {
-            while (t <= seg_end[seg]) {
-                const bool stopped = (seg == 1) ? run_tiles(t, seg_end[seg], std::false_type{})
-                                                : run_tiles(t, seg_end[seg], std::true_type{});
-                if (!stopped) break;
-                // ---- slow path: move the reference of the rows that left the safe range
-                const bool fresh = seen == -INFINITY;
-                const bool move = tmax > 64.f || (fresh && tmax < -32.f && tmax > -INFINITY);
-                const float shift = move ? tmax : 0.f;
-                const float alpha = fresh ? 1.f : fast_exp2(-shift);   // fresh rows hold T = l = 0
-#pragma unroll
-                for (int s = 0; s < 2; ++s) {
-#pragma unroll
-                    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                        for (int rr = 0; rr < 16; ++rr) T[s][dt][rr] *= alpha;
-#pragma unroll
-                    for (int rr = 0; rr < 16; ++rr) X[s][rr] -= shift;
-                }
-                l *= alpha;
-                acc_scale *= alpha;
-                M += shift;
-                seen = fmaxf(seen - shift, tmax - shift);
-                finish_tile();
-                ++t;
-            }
-        }
+        auto run_segment = [&](int t, int t_end, auto masked_tag) {
+            while (t <= t_end && steps(t, t_end, masked_tag)) slow_path();
+        };
+        run_segment(t_lo, mid_lo - 2, std::true_type{});                    // tile t+1 in the masked head
+        run_segment(mid_lo - 1 > t_lo ? mid_lo - 1 : t_lo, t_hi - 2, std::false_type{});   // t+1 unmasked
+        if (t_hi > t_lo) run_segment(t_hi - 1, t_hi - 1, std::true_type{});  // t+1 = diagonal tile
+        // ---- last tile of the round: nothing to overlap with
+        sync_and_refill();
+        load_vf(buf_use);
+        buf_use = next_buf(buf_use);
+        exps();
+        t_gemm();
+        l += (lp[0] + lp[1]) + (lp[2] + lp[3]);
 
         // ---- round end: O_i = (O_i * acc_scale + v2_{i-dlt} * T_i) re-centred on the
         // running maximum, so that the next round starts with x <= 0 for what was seen
