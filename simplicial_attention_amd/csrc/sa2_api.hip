@@ -14,6 +14,7 @@
 #include "sa2_common.hpp"
 #include "sa2_fwd.hpp"
 #include "sa2_fwd_ds.hpp"
+#include "sa2_fwd8.hpp"
 
 namespace {
 
@@ -131,12 +132,18 @@ int sa2_fwd(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, 
             hipLaunchKernelGGL(sa2::fwd_kernel<128>, dim3(grid), dim3(256), 0, s, k);
         else
             hipLaunchKernelGGL(sa2::fwd_kernel<64>, dim3(grid), dim3(256), 0, s, k);
-    } else {
+    } else if (impl && std::strcmp(impl, "ds") == 0) {
         int grid = prob->batch * prob->heads * ((prob->seq_len + 31) / 32);
         if (prob->dim_head == 128)
             hipLaunchKernelGGL(sa2::fwd_ds_kernel<128>, dim3(grid), dim3(256), 0, s, k);
         else
             hipLaunchKernelGGL(sa2::fwd_ds_kernel<64>, dim3(grid), dim3(256), 0, s, k);
+    } else {
+        int grid = prob->batch * prob->heads * ((prob->seq_len + 31) / 32);
+        if (prob->dim_head == 128)
+            hipLaunchKernelGGL(sa2::fwd8_kernel<128>, dim3(grid), dim3(512), 0, s, k);
+        else
+            hipLaunchKernelGGL(sa2::fwd8_kernel<64>, dim3(grid), dim3(512), 0, s, k);
     }
     return after_launch("forward");
 }
