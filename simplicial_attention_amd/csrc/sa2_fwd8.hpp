@@ -7,7 +7,7 @@
 //
 // One workgroup owns 32 query rows of one (batch, head).  In round r wave w handles the
 // offset dlt = i - k = 8r + w; all eight waves walk the same 32-row K1/V1 tiles, which
-// stream through a 3-stage LDS ring (one barrier per tile).  Per (offset, tile):
+// stream through a double-buffered LDS ring two tiles at a time (one barrier per 64 rows).  Per (offset, tile):
 //     S^T = K1 A^T          A = q_i * k2_{i-dlt}   (bf16, built once per offset)
 //     P^T = exp2(S^T scale log2e - M_i)
 //     T^T += V1^T P^T       (V1 fragments through ds_read_b64_tr_b16)
@@ -31,11 +31,13 @@ template <int D>
 struct Fwd8 {
     static constexpr int KS = D / 16;
     static constexpr int DT = D / 32;
+    static constexpr int CT = 2;                      // 32-row tiles per ring stage (per barrier)
     static constexpr int TILE = 32 * tile_pitch<D>(); // K1 tile, read row-major
     static constexpr int VPITCH = tr_pitch<D>();
     static constexpr int VTILE = 32 * VPITCH;         // V1 tile, read through transposed reads only
-    static constexpr int NBUF = 3;
-    static constexpr int STAGE = TILE + VTILE;
+    static constexpr int SUB = TILE + VTILE;          // one K1 tile + one V1 tile
+    static constexpr int STAGE = CT * SUB;
+    static constexpr int NBUF = 2;
     static constexpr int RING = NBUF * STAGE;
     static constexpr int APITCH = D + 4;              // floats per row of the shared accumulator
     static constexpr int ACC = 32 * APITCH * 4;
@@ -47,13 +49,12 @@ struct Fwd8 {
     static constexpr int V2S = K2S + SROWS * tile_pitch<D>();   // v2 rows      [SROWS][pitch]
     static constexpr int LDS = V2S + SROWS * tile_pitch<D>();
     static constexpr int PIECES = 32 * D / 8;         // 16-byte pieces per tile
-    static constexpr int SL = D / 8;                  // d values per slice (8 slices)
 };
 
 template <int D>
 __global__ __launch_bounds__(512) void fwd8_kernel(KParams p) {
     using C = Fwd8<D>;
-    constexpr int KS = C::KS, DT = C::DT, PPR = D / 8, PITCH = tile_pitch<D>();
+    constexpr int KS = C::KS, DT = C::DT, CT = C::CT, PPR = D / 8, PITCH = tile_pitch<D>();
     __shared__ __attribute__((aligned(16))) char lds[C::LDS];
 
     const int N = p.N;
@@ -70,9 +71,7 @@ __global__ __launch_bounds__(512) void fwd8_kernel(KParams p) {
     const int i0 = tile * 32;
     const int i = i0 + c;
     const bool row_ok = i < N;
-    const int ic = row_ok ? i : N - 1;
 
-    const char *qrow = p.q.ptr + b * p.q.sb + (int64_t)ic * p.q.sn + h * p.q.sh;
     const char *k1g = p.k1.ptr + b * p.k1.sb + hk * p.k1.sh;
     const char *v1g = p.v1.ptr + b * p.v1.sb + hk * p.v1.sh;
     const char *k2g = p.k2.ptr + b * p.k2.sb + hk * p.k2.sh;
@@ -81,30 +80,44 @@ __global__ __launch_bounds__(512) void fwd8_kernel(KParams p) {
     const int t_lo = (i0 - p.w1 + 1 > 0 ? i0 - p.w1 + 1 : 0) / 32;
     const int t_hi = i0 / 32;
     const int NT = t_hi - t_lo + 1;
+    const int NC = (NT + CT - 1) / CT;                // ring stages (chunks of CT tiles) per round
     const int nd = p.w2 < i0 + 32 ? p.w2 : i0 + 32;   // offsets that meet at least one valid k
     const int R = (nd + 7) / 8;
-    const int U = R * NT;
+    const int U = R * NC;
     const float c2 = p.scale_log2e;
 
-    // ---- tile staging: the first PIECES threads move one 16-byte piece of K1 and of V1
+    // ---- ring staging: the first PIECES threads move one 16-byte piece of K1 and of V1 per tile
     const bool stager = tid < C::PIECES;
     const int st_row = tid / PPR, st_col = (tid % PPR) * 16;
     const int st_off = st_row * PITCH + st_col;
     const int st_off_v = C::TILE + st_row * C::VPITCH + st_col;
-    u32x4 st_k = {0u, 0u, 0u, 0u}, st_v = {0u, 0u, 0u, 0u};
-    auto issue_loads = [&](int t) {
+    u32x4 st_k[CT], st_v[CT];
+#pragma unroll
+    for (int x = 0; x < CT; ++x) st_k[x] = st_v[x] = (u32x4){0u, 0u, 0u, 0u};
+    int c_load = 0, u_load = 0;                       // chunk (within the round) / running count of the next load
+    auto issue_loads = [&]() {
         if (stager) {
-            int j = 32 * t + st_row;
-            j = j < N ? j : N - 1;
-            st_k = ld_global16(k1g + (int64_t)j * p.k1.sn + st_col);
-            st_v = ld_global16(v1g + (int64_t)j * p.v1.sn + st_col);
+#pragma unroll
+            for (int x = 0; x < CT; ++x) {
+                int t = t_lo + CT * c_load + x;
+                t = t < t_hi ? t : t_hi;              // a missing second tile reloads the diagonal one
+                int j = 32 * t + st_row;
+                j = j < N ? j : N - 1;
+                st_k[x] = ld_global16(k1g + (int64_t)j * p.k1.sn + st_col);
+                st_v[x] = ld_global16(v1g + (int64_t)j * p.v1.sn + st_col);
+            }
         }
+        ++u_load;
+        c_load = (c_load == NC - 1) ? 0 : c_load + 1;
     };
     auto write_stage = [&](int buf) {
         if (stager) {
             char *stage = lds + buf * C::STAGE;
-            *reinterpret_cast<u32x4 *>(stage + st_off) = st_k;
-            *reinterpret_cast<u32x4 *>(stage + st_off_v) = st_v;
+#pragma unroll
+            for (int x = 0; x < CT; ++x) {
+                *reinterpret_cast<u32x4 *>(stage + x * C::SUB + st_off) = st_k[x];
+                *reinterpret_cast<u32x4 *>(stage + x * C::SUB + st_off_v) = st_v[x];
+            }
         }
     };
     const int k_lane = c * PITCH + 16 * hf;          // K1 fragment: row c, pieces 2*kk + hf
@@ -142,20 +155,12 @@ __global__ __launch_bounds__(512) void fwd8_kernel(KParams p) {
     float seen = -INFINITY;    // running maximum of x relative to M; -inf: no valid entry yet
     float l = 0.f;
 
-    int t_load = t_lo, buf_fill = 0, buf_use = 0, u_load = 0;
-    auto advance_load = [&]() {
-        ++u_load;
-        t_load = (t_load == t_hi) ? t_lo : t_load + 1;
-    };
-    auto next_buf = [&](int x) { return x == C::NBUF - 1 ? 0 : x + 1; };
-    issue_loads(t_load);
-    advance_load();
+    // ring protocol: the stage of step u+1 is written right after the barrier of step u (its
+    // buffer was last read in step u-1), from registers loaded during step u-1
+    issue_loads();
     write_stage(0);
-    buf_fill = 1;
-    if (U > 1) {
-        issue_loads(t_load);
-        advance_load();
-    }
+    if (U > 1) issue_loads();
+    int u = 0;                 // running step counter
 
     __syncthreads();           // staged q/k2/v2 rows and the zeroed accumulator are visible
     for (int r = 0; r < R; ++r) {
@@ -178,16 +183,14 @@ __global__ __launch_bounds__(512) void fwd8_kernel(KParams p) {
         f32x16 X;
         float tmax = 0.f;
         u32x2 vf[DT][2][2];
+        const char *stage = lds;
+        // exponentials, row sums and T^T += V1^T P^T for the tile whose logits are in X
         auto finish_tile = [&]() {
             u32x4 pb[2];
 #pragma unroll
             for (int rr = 0; rr < 16; rr += 2) {
-#ifdef WHATIF_NOEXP
-                float p0 = X[rr] * 0.001f, p1 = X[rr + 1] * 0.001f;
-#else
                 float p0 = fast_exp2(X[rr]);
                 float p1 = fast_exp2(X[rr + 1]);
-#endif
                 l += p0 + p1;
                 pb[rr >> 3][(rr & 7) >> 1] = pack_bf16(p0, p1);
             }
@@ -196,112 +199,123 @@ __global__ __launch_bounds__(512) void fwd8_kernel(KParams p) {
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
                     u32x4 v = {vf[dt][k2s][0][0], vf[dt][k2s][0][1], vf[dt][k2s][1][0], vf[dt][k2s][1][1]};
-#ifdef WHATIF_NOMFMA
-                    T[dt][k2s] += as_f32(v[0] ^ pb[k2s][1]);
-#else
                     T[dt] = mfma32(v, pb[k2s], T[dt]);
-#endif
                 }
         };
-        // One pass over tiles [t, t_end].  Returns true if it stopped at tile t because a
-        // row left the safe exponent range (X, tmax, vf of that tile are then still live).
-        auto run_tiles = [&](int &t, int t_end, auto masked_tag) -> bool {
+        // logits of sub-tile x of the current stage -> X (scaled, referenced, masked), tmax;
+        // returns true if some row left the safe exponent range
+        auto logits = [&](int x, int t, auto masked_tag) -> bool {
             constexpr bool MASKED = decltype(masked_tag)::value;
-            for (; t <= t_end; ++t) {
-#ifndef WHATIF_NOBARRIER
-                __syncthreads();
-#endif
-#ifndef WHATIF_NOSTAGE
-                if (u_load - 1 > r * NT + (t - t_lo)) {
-                    write_stage(buf_fill);
-                    buf_fill = next_buf(buf_fill);
+            const char *kbase = stage + x * C::SUB + k_lane;
+            const char *vbase = stage + x * C::SUB + v_lane;
+            X = zero16();
+            u32x4 kf[KS];
+#pragma unroll
+            for (int kk = 0; kk < KS; ++kk) kf[kk] = ld_lds16(kbase + 32 * kk);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int kk = 0; kk < KS; ++kk) X = mfma32(kf[kk], A[kk], X);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int k2s = 0; k2s < 2; ++k2s) {
+                    vf[dt][k2s][0] = lds_read_tr<D, C::VPITCH>(vbase, 16 * k2s, 32 * dt);
+                    vf[dt][k2s][1] = lds_read_tr<D, C::VPITCH>(vbase, 16 * k2s + 8, 32 * dt);
                 }
-                if (u_load < U) {
-                    issue_loads(t_load);
-                    advance_load();
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int rr = 0; rr < 16; ++rr) X[rr] = X[rr] * c2 - M;
+            if constexpr (MASKED) {
+#pragma unroll
+                for (int rr = 0; rr < 16; ++rr) {
+                    int j = 32 * t + 8 * (rr >> 2) + 4 * hf + (rr & 3);
+                    bool ok = col_ok && (j <= i) && (j + p.w1 > i);
+                    X[rr] = ok ? X[rr] : -INFINITY;
                 }
-#endif
-                const char *kbase = lds + buf_use * C::STAGE + k_lane;
-                const char *vbase = lds + buf_use * C::STAGE + v_lane;
-                buf_use = next_buf(buf_use);
+            }
+            tmax = X[0];
+#pragma unroll
+            for (int rr = 1; rr < 16; ++rr) tmax = fmaxf(tmax, X[rr]);
+            auto sw = __builtin_amdgcn_permlane32_swap(as_u32(tmax), as_u32(tmax), false, false);
+            tmax = fmaxf(as_f32(sw[0]), as_f32(sw[1]));
+            return wave_any(tmax > 64.f || (seen == -INFINITY && tmax < -32.f && tmax > -INFINITY));
+        };
+        // slow path (kept outside the hot loop on purpose): move the reference of the rows
+        // that left the safe range and rescale what T and l already hold
+        auto move_reference = [&]() {
+            const bool fresh = seen == -INFINITY;
+            const bool move = tmax > 64.f || (fresh && tmax < -32.f && tmax > -INFINITY);
+            const float shift = move ? tmax : 0.f;
+            const float alpha = fresh ? 1.f : fast_exp2(-shift);
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int rr = 0; rr < 16; ++rr) T[dt][rr] *= alpha;
+#pragma unroll
+            for (int rr = 0; rr < 16; ++rr) X[rr] -= shift;
+            l *= alpha;
+            M += shift;
+            seen -= shift;
+            tmax -= shift;
+        };
+        // barrier + refill of the ring behind the stage that becomes current
+        auto sync_stage = [&]() {
+            __syncthreads();
+            if (u_load - 1 > u) write_stage((u + 1) & 1);
+            if (u_load < U) issue_loads();
+            stage = lds + (u & 1) * C::STAGE;
+            ++u;
+        };
+        // Runs chunks cc .. cc_end.  Returns true if it stopped inside chunk cc at sub-tile
+        // `stop_x` because the logits in X left the safe range (nothing of that sub-tile
+        // has been accumulated yet).
+        int stop_x = 0;
+        auto run_chunks = [&](int &cc, int cc_end, auto masked_tag) -> bool {
+            constexpr bool MASKED = decltype(masked_tag)::value;
+            for (; cc <= cc_end; ++cc) {
+                sync_stage();
                 if (!wave_on) continue;
-
-                X = zero16();
-#ifdef WHATIF_NOLDS
-                const char *kb2 = lds + k_lane, *vb2 = lds + v_lane;
-#else
-                const char *kb2 = kbase, *vb2 = vbase;
-#endif
-#pragma unroll
-                for (int kk = 0; kk < KS; ++kk) {
-#ifdef WHATIF_NOMFMA
-                    u32x4 kf_ = ld_lds16(kb2 + 32 * kk);
-                    X[kk] += as_f32(kf_[0] ^ A[kk][1]);
-                    X[kk + 8] += as_f32(kf_[2] ^ A[kk][3]);
-#else
-                    X = mfma32(ld_lds16(kb2 + 32 * kk), A[kk], X);
-#endif
-                }
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                    for (int k2s = 0; k2s < 2; ++k2s) {
-                        vf[dt][k2s][0] = lds_read_tr<D, C::VPITCH>(vb2, 16 * k2s, 32 * dt);
-                        vf[dt][k2s][1] = lds_read_tr<D, C::VPITCH>(vb2, 16 * k2s + 8, 32 * dt);
+#pragma nounroll
+                for (int x = 0; x < CT; ++x) {
+                    const int t = t_lo + CT * cc + x;
+                    if (MASKED && t > t_hi) break;
+                    if (logits(x, t, masked_tag)) {
+                        stop_x = x;
+                        return true;
                     }
-#pragma unroll
-                for (int rr = 0; rr < 16; ++rr) X[rr] = X[rr] * c2 - M;
-                if constexpr (MASKED) {
-#pragma unroll
-                    for (int rr = 0; rr < 16; ++rr) {
-                        int j = 32 * t + 8 * (rr >> 2) + 4 * hf + (rr & 3);
-                        bool ok = col_ok && (j <= i) && (j + p.w1 > i);
-                        X[rr] = ok ? X[rr] : -INFINITY;
-                    }
+                    seen = fmaxf(seen, tmax);
+                    finish_tile();
                 }
-                tmax = X[0];
-#pragma unroll
-                for (int rr = 1; rr < 16; ++rr) tmax = fmaxf(tmax, X[rr]);
-                {
-                    auto sw = __builtin_amdgcn_permlane32_swap(as_u32(tmax), as_u32(tmax), false, false);
-                    tmax = fmaxf(as_f32(sw[0]), as_f32(sw[1]));
-                }
-                if (wave_any(tmax > 64.f || (seen == -INFINITY && tmax < -32.f && tmax > -INFINITY))) return true;
-                seen = fmaxf(seen, tmax);
-                finish_tile();
             }
             return false;
         };
 
-        // tiles [t_lo, t_hi] = masked head | unmasked middle | masked tail (the diagonal)
-        int mid_lo = (i0 + 31 - p.w1 >= 0) ? (i0 + 31 - p.w1) / 32 + 1 : t_lo;
+        // chunks of the window: masked head | unmasked middle | masked tail (holds the diagonal)
+        int mid_lo = (i0 + 31 - p.w1 >= 0) ? (i0 + 31 - p.w1) / 32 + 1 : t_lo;   // first unmasked tile
         if (any_bad) mid_lo = t_hi;
         mid_lo = mid_lo > t_hi ? t_hi : mid_lo;
-        const int seg_end[3] = {mid_lo - 1, t_hi - 1, t_hi};
-        int t = t_lo;
+        const int c_mid_lo = (mid_lo - t_lo + CT - 1) / CT;         // first chunk made of unmasked tiles only
+        const int c_mid_hi = (t_hi - t_lo) / CT - 1;                // last chunk that ends before the diagonal tile
+        const int seg_end[3] = {c_mid_lo - 1, c_mid_hi, NC - 1};
+        int cc = 0;
 #pragma unroll
         for (int seg = 0; seg < 3; ++seg) {
-            while (t <= seg_end[seg]) {
-                const bool stopped = (seg == 1) ? run_tiles(t, seg_end[seg], std::false_type{})
-                                                : run_tiles(t, seg_end[seg], std::true_type{});
+            while (cc <= seg_end[seg]) {
+                const bool stopped = (seg == 1) ? run_chunks(cc, seg_end[seg], std::false_type{})
+                                                : run_chunks(cc, seg_end[seg], std::true_type{});
                 if (!stopped) break;
-                // slow path (outside the hot loop on purpose): move the reference of the rows
-                // that left the safe range and rescale what T and l already hold
-                const bool fresh = seen == -INFINITY;
-                const bool move = tmax > 64.f || (fresh && tmax < -32.f && tmax > -INFINITY);
-                const float shift = move ? tmax : 0.f;
-                const float alpha = fresh ? 1.f : fast_exp2(-shift);
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                    for (int rr = 0; rr < 16; ++rr) T[dt][rr] *= alpha;
-#pragma unroll
-                for (int rr = 0; rr < 16; ++rr) X[rr] -= shift;
-                l *= alpha;
-                M += shift;
-                seen = fmaxf(seen - shift, tmax - shift);
+                // finish chunk cc on the slow path
+                move_reference();
+                seen = fmaxf(seen, tmax);
                 finish_tile();
-                ++t;
+                for (int x = stop_x + 1; x < CT; ++x) {
+                    const int t = t_lo + CT * cc + x;
+                    if (t > t_hi) break;
+                    if (logits(x, t, std::true_type{})) move_reference();
+                    seen = fmaxf(seen, tmax);
+                    finish_tile();
+                }
+                ++cc;
             }
         }
 
@@ -346,9 +360,8 @@ __global__ __launch_bounds__(512) void fwd8_kernel(KParams p) {
                 *reinterpret_cast<float4 *>(dst + 4) = a1;
             };
             for (int ph = 0; ph < 8; ++ph) {
-                const int slice = (wave + ph) & 7;
                 if constexpr (DT == 4) {
-                    switch (slice) {
+                    switch ((wave + ph) & 7) {
                         case 0: add_slice(std::integral_constant<int, 0>{}, ph == 0); break;
                         case 1: add_slice(std::integral_constant<int, 1>{}, ph == 0); break;
                         case 2: add_slice(std::integral_constant<int, 2>{}, ph == 0); break;
