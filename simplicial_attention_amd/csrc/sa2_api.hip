@@ -10,6 +10,7 @@
 #include <cstring>
 
 #include "sa2_bwd.hpp"
+#include "sa2_bwd_q8.hpp"
 #include "sa2_bwd_qk2.hpp"
 #include "sa2_common.hpp"
 #include "sa2_fwd.hpp"
@@ -227,7 +228,17 @@ int sa2_bwd_dq_dkv2(const sa2_problem *prob, const sa2_tensor *q, const sa2_tens
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
     const int grid = prob->batch * prob->heads * ((prob->seq_len + 31) / 32);
     const int w2max = qk2_w2max(prob->w2);
-    if (prob->dim_head == 128 && w2max == 32)
+    // offsets up to 32: two eight-wave passes (dq + dk2, then dv2); wider second windows (or
+    // SA2_BWD_QK2_IMPL=fused) take the fused four-wave kernel
+    const char *impl = std::getenv("SA2_BWD_QK2_IMPL");
+    const bool fused = w2max > 32 || (impl && std::strcmp(impl, "fused") == 0);
+    if (!fused && prob->dim_head == 128) {
+        hipLaunchKernelGGL((sa2::bwd_q8_kernel<128, true>), dim3(grid), dim3(512), 0, s, k, ws);
+        hipLaunchKernelGGL((sa2::bwd_q8_kernel<128, false>), dim3(grid), dim3(512), 0, s, k, ws);
+    } else if (!fused) {
+        hipLaunchKernelGGL((sa2::bwd_q8_kernel<64, true>), dim3(grid), dim3(512), 0, s, k, ws);
+        hipLaunchKernelGGL((sa2::bwd_q8_kernel<64, false>), dim3(grid), dim3(512), 0, s, k, ws);
+    } else if (prob->dim_head == 128 && w2max == 32)
         hipLaunchKernelGGL((sa2::bwd_qk2_kernel<128, 32>), dim3(grid), dim3(256), 0, s, k, ws);
     else if (prob->dim_head == 128)
         hipLaunchKernelGGL((sa2::bwd_qk2_kernel<128, 64>), dim3(grid), dim3(256), 0, s, k, ws);
