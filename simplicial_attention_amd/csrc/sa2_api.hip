@@ -10,6 +10,7 @@
 #include <cstring>
 
 #include "sa2_bwd.hpp"
+#include "sa2_bwd_kv8.hpp"
 #include "sa2_bwd_q8.hpp"
 #include "sa2_bwd_qk2.hpp"
 #include "sa2_common.hpp"
@@ -266,9 +267,22 @@ int sa2_bwd_dkv1(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor 
     SA2_TRY(check_tensor(dv1, "dv1"));
     k.dk1 = dev(dk1);
     k.dv1 = dev(dv1);
+#ifdef SA2_TIMING
+    k.dq = dev(dk1);
+#endif
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
     int grid = prob->batch * prob->kv_heads * ((prob->seq_len + 127) / 128);
-    if (prob->dim_head == 128)
+    // offsets up to 32: two eight-wave passes (dk1, then dv1); wider second windows (or
+    // SA2_BWD_KV1_IMPL=fused) take the fused four-wave kernel
+    const char *impl = std::getenv("SA2_BWD_KV1_IMPL");
+    const bool fused = prob->w2 > 32 || (impl && std::strcmp(impl, "fused") == 0);
+    if (!fused && prob->dim_head == 128) {
+        hipLaunchKernelGGL((sa2::bwd_kv8_kernel<128, true>), dim3(grid), dim3(512), 0, s, k);
+        hipLaunchKernelGGL((sa2::bwd_kv8_kernel<128, false>), dim3(grid), dim3(512), 0, s, k);
+    } else if (!fused) {
+        hipLaunchKernelGGL((sa2::bwd_kv8_kernel<64, true>), dim3(grid), dim3(512), 0, s, k);
+        hipLaunchKernelGGL((sa2::bwd_kv8_kernel<64, false>), dim3(grid), dim3(512), 0, s, k);
+    } else if (prob->dim_head == 128)
         hipLaunchKernelGGL(sa2::bwd_dkv1_kernel<128>, dim3(grid), dim3(256), 0, s, k);
     else
         hipLaunchKernelGGL(sa2::bwd_dkv1_kernel<64>, dim3(grid), dim3(256), 0, s, k);

@@ -1,0 +1,351 @@
+// Backward kernels for dK1 and for dV1, eight-wave variant (two waves per SIMD).
+//
+// Workgroup = 128 rows j of one (batch, kv head).  The eight waves are four 32-row slabs
+// of j times two step groups: the workgroup walks pairs of "steps" (query head of the
+// group, 32-row query tile, offset dlt); of a pair, the waves of group 0 take the even
+// offset and the waves of group 1 the odd one.  The q/do rows of a query tile and the 63
+// k2/v2 rows its offsets (at most 32) can reach are staged in LDS once per tile; from
+// them the 512 threads build A = q*k2 and B = do*v2 of both steps once per barrier.  A fused kernel (dK1 and dV1
+// accumulators, K1 and V1 fragments) needs a whole SIMD's registers for one wave, and one
+// wave cannot overlap its own MFMA and VALU work; so there are two passes that fit two
+// waves per SIMD:
+//   pass DK (DK = true):   S = A K1^T, dP = B V1^T, dS = P (dP - delta),  dK1^T += A^T dS
+//   pass DV (DK = false):  S = A K1^T,                                     dV1^T += B^T P
+// with P = exp2(S scale log2e - lse).  Row-major tiles feed S and dP, copies with the
+// pitch of the transposed reads feed the accumulating products.  The two groups of a
+// slab hold partial sums that are added once, through LDS, at the end.
+#pragma once
+
+#include "sa2_common.hpp"
+#include "sa2_fwd_ds.hpp"
+
+namespace sa2 {
+
+template <int D, bool DK>
+struct Kv8Cfg {
+    static constexpr int PITCH = tile_pitch<D>();
+    static constexpr int TILE = 32 * PITCH;
+    static constexpr int TPITCH = tr_pitch<D>();
+    static constexpr int TRT = 32 * TPITCH;
+    // step buffer: DK: [A row-major][A transposed-read copy][B row-major][lse][delta]
+    //              DV: [A row-major][B transposed-read][lse]
+    static constexpr int AS = 0;
+    static constexpr int TR = TILE;                   // the tile read through transposed reads
+    static constexpr int BS = TILE + TRT;             // DK only
+    static constexpr int LSE = DK ? 2 * TILE + TRT : TILE + TRT;
+    static constexpr int DEL = LSE + 32 * 4;
+    static constexpr int STEP = DEL + 32 * 4;
+    static constexpr int PAIR = 2 * STEP;
+    static constexpr int TILES = 2 * PAIR;            // double-buffered pairs
+    // staged rows of the current query tile (unpadded, read lane-linear by the builders)
+    static constexpr int HALO = 31;
+    static constexpr int KROWS = 32 + HALO;           // k in [32 it - 31, 32 it + 31]
+    static constexpr int RP = 2 * D;                  // bytes per staged row
+    static constexpr int QS = TILES;
+    static constexpr int DOS = QS + 32 * RP;
+    static constexpr int K2S = DOS + 32 * RP;
+    static constexpr int V2S = K2S + KROWS * RP;
+    static constexpr int LSES = V2S + KROWS * RP;     // 32 floats lse * log2e, 32 floats delta
+    static constexpr int LDS = LSES + 64 * 4;
+    static constexpr int NROWP = (64 + 2 * KROWS) * (D / 8);        // 16-byte pieces of the staged rows
+    static constexpr int RPT = (NROWP + 511) / 512;                 // ... per thread
+    static constexpr int RPITCH = D + 4;              // floats per row of the final reduction
+    static constexpr int LPT = 32 * D / 8 / 256;      // 16-byte pieces per thread and tensor
+    static_assert(128 * RPITCH * 4 <= TILES, "final reduction must fit the tile buffers");
+};
+
+template <int D, bool DK>
+__global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
+    constexpr int KS = D / 16, DT = D / 32, PPR = D / 8;
+    using L = Kv8Cfg<D, DK>;
+    constexpr int PITCH = L::PITCH;
+    __shared__ __attribute__((aligned(16))) char lds[L::LDS];
+
+    const int N = p.N;
+    const int ntile = (N + 127) / 128;
+    const int item = xcd_contiguous(blockIdx.x, gridDim.x);
+    const int tile = item % ntile;
+    const int bh = item / ntile;
+    const int hk = bh % p.HK, b = bh / p.HK;
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63;
+    const int slab = wave & 3, pg = wave >> 2;
+    const int c = lane & 31, hf = lane >> 5;
+    const int j0 = tile * 128;
+    const int jw = j0 + 32 * slab;
+    const int j = jw + c;
+    const bool j_ok = j < N;
+    const int jc = j_ok ? j : N - 1;
+
+    const char *k2g = p.k2.ptr + b * p.k2.sb + hk * p.k2.sh;
+    const char *v2g = p.v2.ptr + b * p.v2.sb + hk * p.v2.sh;
+
+    u32x4 k1f[KS];
+    u32x4 v1f[DK ? KS : 1];
+    {
+        const char *k1row = p.k1.ptr + b * p.k1.sb + (int64_t)jc * p.k1.sn + hk * p.k1.sh;
+        const char *v1row = p.v1.ptr + b * p.v1.sb + (int64_t)jc * p.v1.sn + hk * p.v1.sh;
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk) {
+            k1f[kk] = ld_global16(k1row + (16 * kk + 8 * hf) * 2);
+            if constexpr (DK) v1f[kk] = ld_global16(v1row + (16 * kk + 8 * hf) * 2);
+        }
+    }
+    f32x16 acc[DT];
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt) acc[dt] = zero16();
+#ifdef SA2_TIMING
+    long long t_acc[6] = {0, 0, 0, 0, 0, 0};
+    long long t_last = __builtin_amdgcn_s_memtime();
+#define TS(k)                                             \
+    {                                                     \
+        __builtin_amdgcn_sched_barrier(0);                \
+        const long long t_now = __builtin_amdgcn_s_memtime(); \
+        t_acc[k] += t_now - t_last;                       \
+        t_last = t_now;                                   \
+        __builtin_amdgcn_sched_barrier(0);                \
+    }
+#else
+#define TS(k)
+#endif
+
+    const int it_begin = j0 / 32;
+    const int last_i = (j0 + 127 + p.w1 - 1 < N - 1) ? j0 + 127 + p.w1 - 1 : N - 1;
+    const int it_end = last_i / 32;
+    const bool wave_active = jw < N;
+    const int wit_lo = jw / 32;
+    const int wit_hi = ((jw + 31 + p.w1 - 1 < N - 1) ? jw + 31 + p.w1 - 1 : N - 1) / 32;
+    const float c2 = p.scale_log2e;
+    const int r_lane = c * PITCH + 16 * hf;
+    const int t_lane = L::TR + tr_lane_off<D, L::TPITCH>(lane);
+
+    // ---- pair iterator (g, it, m): offsets 2m and 2m+1 of query tile `it`, query head g of the group
+    struct Pair {
+        int g, it, m;
+    };
+    auto dmax_of = [&](int it) { return (p.w2 - 1 < 32 * it + 31) ? p.w2 - 1 : 32 * it + 31; };
+    auto next_pair = [&](Pair &s) {
+        if (2 * (++s.m) > dmax_of(s.it)) {
+            s.m = 0;
+            if (++s.it > it_end) {
+                s.it = it_begin;
+                ++s.g;
+            }
+        }
+    };
+    int npairs = 0;
+    for (int it = it_begin; it <= it_end; ++it) npairs += dmax_of(it) / 2 + 1;
+    npairs *= p.G;
+
+    // ---- row staging: per (query head, query tile) the q/do rows and the k2/v2 rows go
+    // global -> registers (a whole tile ahead) -> LDS
+    u32x4 rows[L::RPT];
+    float r_lse = 0.f, r_del = 0.f;
+    auto issue_rows = [&](const Pair &s) {
+        const int h = hk * p.G + s.g;
+        const char *qg = p.q.ptr + b * p.q.sb + h * p.q.sh;
+        const char *dog = p.dout.ptr + b * p.dout.sb + h * p.dout.sh;
+#pragma unroll
+        for (int x = 0; x < L::RPT; ++x) {
+            const int pc = x * 512 + tid;
+            if (pc >= L::NROWP) break;
+            const int row = pc / PPR, col = (pc % PPR) * 16;
+            const char *src;
+            if (row < 64) {
+                int i = 32 * s.it + (row & 31);
+                i = i < N ? i : N - 1;
+                src = (row < 32 ? qg + (int64_t)i * p.q.sn : dog + (int64_t)i * p.dout.sn);
+            } else {
+                const int rk = row - 64;
+                int kr = 32 * s.it - L::HALO + (rk < L::KROWS ? rk : rk - L::KROWS);
+                kr = kr < 0 ? 0 : (kr < N ? kr : N - 1);
+                src = (rk < L::KROWS ? k2g + (int64_t)kr * p.k2.sn : v2g + (int64_t)kr * p.v2.sn);
+            }
+            rows[x] = ld_global16(src + col);
+        }
+        if (tid < 32) {
+            const int i = 32 * s.it + tid;
+            const int icl = i < N ? i : N - 1;
+            r_lse = p.lse[((int64_t)b * p.H + h) * N + icl] * kLog2e;
+            if constexpr (DK) r_del = p.delta[((int64_t)b * p.H + h) * N + icl];
+        }
+    };
+    auto write_rows = [&]() {
+#pragma unroll
+        for (int x = 0; x < L::RPT; ++x) {
+            const int pc = x * 512 + tid;
+            if (pc >= L::NROWP) break;
+            *reinterpret_cast<u32x4 *>(lds + L::QS + pc * 16) = rows[x];     // q, do, k2, v2 rows are contiguous
+        }
+        if (tid < 32) {
+            reinterpret_cast<float *>(lds + L::LSES)[tid] = r_lse;
+            if constexpr (DK) reinterpret_cast<float *>(lds + L::LSES)[32 + tid] = r_del;
+        }
+    };
+
+    // ---- operand build: threads 0-255 build the even step of a pair, 256-511 the odd one
+    const int sub = tid >> 8, t8 = tid & 255;
+    auto build = [&](const Pair &s, int buf) {
+        char *stage = lds + buf * L::PAIR + sub * L::STEP;
+        const int dlt = 2 * s.m + sub;
+        const bool dead = dlt > dmax_of(s.it);        // odd number of offsets: the last pair is half empty
+        const int dl = dead ? 0 : dlt;
+#pragma unroll
+        for (int x = 0; x < L::LPT; ++x) {
+            const int pc = x * 256 + t8;
+            const int row = pc / PPR, col = (pc % PPR) * 16;
+            const int krow = row - dl + L::HALO;
+            const u32x4 a = mul_bf16x8(ld_lds16(lds + L::QS + row * L::RP + col), ld_lds16(lds + L::K2S + krow * L::RP + col));
+            *reinterpret_cast<u32x4 *>(stage + L::AS + row * PITCH + col) = a;
+            if constexpr (DK) *reinterpret_cast<u32x4 *>(stage + L::TR + row * L::TPITCH + col) = a;
+            __builtin_amdgcn_sched_barrier(0);        // one product at a time: keeps the build's registers few
+            const u32x4 bb = mul_bf16x8(ld_lds16(lds + L::DOS + row * L::RP + col), ld_lds16(lds + L::V2S + krow * L::RP + col));
+            *reinterpret_cast<u32x4 *>(stage + (DK ? L::BS + row * PITCH : L::TR + row * L::TPITCH) + col) = bb;
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (t8 < 32) {
+            const int i = 32 * s.it + t8;
+            const bool valid = !dead && i < N && i - dlt >= 0;
+            reinterpret_cast<float *>(stage + L::LSE)[t8] = valid ? reinterpret_cast<const float *>(lds + L::LSES)[t8] : INFINITY;
+            if constexpr (DK) reinterpret_cast<float *>(stage + L::DEL)[t8] = valid ? reinterpret_cast<const float *>(lds + L::LSES)[32 + t8] : 0.f;
+        }
+    };
+    auto next_tile = [&](Pair &s) {      // first pair of the next (query head, query tile)
+        s.m = 0;
+        if (++s.it > it_end) {
+            s.it = it_begin;
+            ++s.g;
+        }
+    };
+
+    Pair nb = {0, it_begin, 0};   // next pair to build
+    Pair cur = {0, it_begin, 0};  // pair being computed
+    Pair rw = {0, it_begin, 0};   // query tile whose rows are loaded next
+    issue_rows(rw);
+    next_tile(rw);
+    write_rows();
+    if (rw.g < p.G) issue_rows(rw);
+    __syncthreads();
+    build(nb, 0);
+    next_pair(nb);
+
+    for (int s = 0; s < npairs; ++s) {
+        __syncthreads();
+        TS(0);
+        if (s + 1 < npairs) {
+            if (nb.m == 0) {
+                // the next pair opens a new query tile: its rows replace the staged ones
+                // (all builds from the old rows ended before the barrier above)
+                write_rows();
+                next_tile(rw);
+                if (rw.g < p.G) issue_rows(rw);
+                __syncthreads();
+            }
+            TS(1);
+            build(nb, (s + 1) & 1);
+            next_pair(nb);
+        }
+        TS(2);
+        const char *buf = lds + (s & 1) * L::PAIR + pg * L::STEP;
+        const int it = cur.it;
+        next_pair(cur);
+        if (!wave_active || it < wit_lo || it > wit_hi) continue;
+
+        // ---- S[i,j] (and dP[i,j]): rows = query rows of the tile, column = j
+        f32x16 X = zero16();
+#pragma unroll
+        for (int kk = 0; kk < KS; ++kk) X = mfma32(ld_lds16(buf + L::AS + r_lane + 32 * kk), k1f[kk], X);
+        f32x16 dP;
+        if constexpr (DK) {
+            dP = zero16();
+#pragma unroll
+            for (int kk = 0; kk < KS; ++kk) dP = mfma32(ld_lds16(buf + L::BS + r_lane + 32 * kk), v1f[kk], dP);
+        }
+#pragma unroll
+        for (int a4 = 0; a4 < 4; ++a4) {
+            const float4 l4 = *reinterpret_cast<const float4 *>(buf + L::LSE + (8 * a4 + 4 * hf) * 4);
+            X[4 * a4] = X[4 * a4] * c2 - l4.x;
+            X[4 * a4 + 1] = X[4 * a4 + 1] * c2 - l4.y;
+            X[4 * a4 + 2] = X[4 * a4 + 2] * c2 - l4.z;
+            X[4 * a4 + 3] = X[4 * a4 + 3] * c2 - l4.w;
+            if constexpr (DK) {
+                const float4 d4 = *reinterpret_cast<const float4 *>(buf + L::DEL + (8 * a4 + 4 * hf) * 4);
+                dP[4 * a4] -= d4.x;
+                dP[4 * a4 + 1] -= d4.y;
+                dP[4 * a4 + 2] -= d4.z;
+                dP[4 * a4 + 3] -= d4.w;
+            }
+        }
+        TS(3);
+        const bool full = (jw + 31 <= 32 * it) && (jw + p.w1 > 32 * it + 31);
+        if (!full) {
+            const int base = 32 * it + 4 * hf - j;   // i - j for register 0
+#pragma unroll
+            for (int rr = 0; rr < 16; ++rr) {
+                const bool ok = (unsigned)(base + 8 * (rr >> 2) + (rr & 3)) < (unsigned)p.w1;
+                X[rr] = ok ? X[rr] : -INFINITY;
+            }
+        }
+        u32x4 pb[2];
+#pragma unroll
+        for (int rr = 0; rr < 16; rr += 2) {
+            float p0 = fast_exp2(X[rr]);
+            float p1 = fast_exp2(X[rr + 1]);
+            if constexpr (DK) {
+                p0 *= dP[rr];
+                p1 *= dP[rr + 1];
+            }
+            pb[rr >> 3][(rr & 7) >> 1] = pack_bf16(p0, p1);
+        }
+        TS(4);
+#pragma unroll
+        for (int k2s = 0; k2s < 2; ++k2s)
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) {
+                u32x2 lo2 = lds_read_tr<D, L::TPITCH>(buf + t_lane, 16 * k2s, 32 * dt);
+                u32x2 hi2 = lds_read_tr<D, L::TPITCH>(buf + t_lane, 16 * k2s + 8, 32 * dt);
+                u32x4 fr = {lo2[0], lo2[1], hi2[0], hi2[1]};
+                acc[dt] = mfma32(fr, pb[k2s], acc[dt]);
+            }
+        TS(5);
+    }
+
+#ifdef SA2_TIMING
+    if (item == (int)gridDim.x / 2 + 3 && lane == 0) {
+        long long *dbg = reinterpret_cast<long long *>(p.dq.ptr) + (DK ? 0 : 64);
+        for (int k = 0; k < 6; ++k) dbg[wave * 8 + k] = t_acc[k];
+        dbg[wave * 8 + 6] = npairs;
+    }
+#endif
+#undef TS
+    // ---- add the two groups of every slab and store
+    __syncthreads();
+    float *red = reinterpret_cast<float *>(lds) + (32 * slab + c) * L::RPITCH + 16 * hf;
+    if (pg == 1) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4)
+                *reinterpret_cast<float4 *>(red + 32 * dt + 4 * r4) =
+                    make_float4(acc[dt][4 * r4], acc[dt][4 * r4 + 1], acc[dt][4 * r4 + 2], acc[dt][4 * r4 + 3]);
+    }
+    __syncthreads();
+    if (pg == 1 || !j_ok) return;
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+            const float4 a = *reinterpret_cast<const float4 *>(red + 32 * dt + 4 * r4);
+            acc[dt][4 * r4] += a.x;
+            acc[dt][4 * r4 + 1] += a.y;
+            acc[dt][4 * r4 + 2] += a.z;
+            acc[dt][4 * r4 + 3] += a.w;
+        }
+    if constexpr (DK)
+        store_row<DT>(p.dk1.ptr + b * p.dk1.sb + (int64_t)j * p.dk1.sn + hk * p.dk1.sh + 16 * hf * 2, acc, p.scale);
+    else
+        store_row<DT>(p.dv1.ptr + b * p.dv1.sb + (int64_t)j * p.dv1.sn + hk * p.dv1.sh + 16 * hf * 2, acc, 1.f);
+}
+
+}  // namespace sa2

@@ -149,6 +149,20 @@ __global__ __launch_bounds__(512) void fwd8_kernel(KParams p) {
         }
     }
 
+#ifdef SA2_TIMING
+    long long t_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    long long t_last = __builtin_amdgcn_s_memtime();
+#define TS(k)                                                 \
+    {                                                         \
+        __builtin_amdgcn_sched_barrier(0);                    \
+        const long long t_now = __builtin_amdgcn_s_memtime(); \
+        t_acc[k] += t_now - t_last;                           \
+        t_last = t_now;                                       \
+        __builtin_amdgcn_sched_barrier(0);                    \
+    }
+#else
+#define TS(k)
+#endif
     f32x16 T[DT];
     u32x4 A[KS];
     float M = 0.f;             // private reference (log2 domain); meaningless while `seen` is -inf
@@ -180,6 +194,7 @@ __global__ __launch_bounds__(512) void fwd8_kernel(KParams p) {
             for (int dt = 0; dt < DT; ++dt) T[dt] = zero16();
         }
 
+        TS(5);
         f32x16 X;
         float tmax = 0.f;
         u32x2 vf[DT][2][2];
@@ -260,11 +275,14 @@ __global__ __launch_bounds__(512) void fwd8_kernel(KParams p) {
         };
         // barrier + refill of the ring behind the stage that becomes current
         auto sync_stage = [&]() {
+            TS(3);
             __syncthreads();
+            TS(0);
             if (u_load - 1 > u) write_stage((u + 1) & 1);
             if (u_load < U) issue_loads();
             stage = lds + (u & 1) * C::STAGE;
             ++u;
+            TS(1);
         };
         // Runs chunks cc .. cc_end.  Returns true if it stopped inside chunk cc at sub-tile
         // `stop_x` because the logits in X left the safe range (nothing of that sub-tile
@@ -284,6 +302,7 @@ __global__ __launch_bounds__(512) void fwd8_kernel(KParams p) {
                         return true;
                     }
                     seen = fmaxf(seen, tmax);
+                    TS(2);
                     finish_tile();
                 }
             }
@@ -320,6 +339,7 @@ __global__ __launch_bounds__(512) void fwd8_kernel(KParams p) {
         }
 
         // ---- round end: agree on the common reference, add v2 * T into the shared rows
+        TS(3);
         {
             const bool fresh = seen == -INFINITY;
             if (hf == 0) xm[wave * 32 + c] = fresh ? -INFINITY : M + seen;
@@ -385,7 +405,18 @@ __global__ __launch_bounds__(512) void fwd8_kernel(KParams p) {
                 __syncthreads();
             }
         }
+        TS(4);
     }
+#ifdef SA2_TIMING
+    const bool timed = item == (int)gridDim.x / 2 + 3 && p.o_lo.ptr;
+    if (timed && lane == 0) {
+        long long *dbg = reinterpret_cast<long long *>(p.o_lo.ptr + b * p.o_lo.sb + (int64_t)(i0 + wave) * p.o_lo.sn + h * p.o_lo.sh);
+        for (int k = 0; k < 6; ++k) dbg[k] = t_acc[k];
+        dbg[6] = U;
+        dbg[7] = R;
+    }
+#endif
+#undef TS
 
     // ---- output: O = acc_sh / L with L = sum_w l_w 2^(M_w - Mc)
     {
@@ -410,6 +441,9 @@ __global__ __launch_bounds__(512) void fwd8_kernel(KParams p) {
         const float *src = acc_sh + row * C::APITCH + seg * SEG;
         char *orow = p.o.ptr + b * p.o.sb + (int64_t)ir * p.o.sn + h * p.o.sh + seg * SEG * 2;
         char *rrow = p.o_lo.ptr ? p.o_lo.ptr + b * p.o_lo.sb + (int64_t)ir * p.o_lo.sn + h * p.o_lo.sh + seg * SEG * 2 : nullptr;
+#ifdef SA2_TIMING
+        if (timed) rrow = nullptr;
+#endif
         float o[SEG];
 #pragma unroll
         for (int x = 0; x < SEG; x += 4) {
