@@ -69,7 +69,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     const int hk = bh % p.HK, b = bh / p.HK;
 
     const int tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63;
+    const int wave = wave_index(), lane = tid & 63;
     const int slab = wave & 3, pg = wave >> 2;
     const int c = lane & 31, hf = lane >> 5;
     const int j0 = tile * 128;
@@ -258,6 +258,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
         for (int kk = 0; kk < KS; ++kk) X = mfma32(ld_lds16(buf + L::AS + r_lane + 32 * kk), k1f[kk], X);
         f32x16 dP;
         if constexpr (DK) {
+            __builtin_amdgcn_sched_barrier(0);        // keeps the two sets of fragments from being live together
             dP = zero16();
 #pragma unroll
             for (int kk = 0; kk < KS; ++kk) dP = mfma32(ld_lds16(buf + L::BS + r_lane + 32 * kk), v1f[kk], dP);

@@ -96,7 +96,7 @@ __global__ __launch_bounds__(512) void bwd_q8_kernel(KParams p, float *ws) {
     const int hk = h / p.G;
 
     const int tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63;
+    const int wave = wave_index(), lane = tid & 63;
     const int c = lane & 31, hf = lane >> 5;
     const int i0 = tile * 32;
     const int i = i0 + c;

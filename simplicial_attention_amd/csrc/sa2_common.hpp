@@ -66,6 +66,30 @@ __device__ __forceinline__ u32x4 mul_bf16x8(u32x4 a, u32x4 b) {
     return r;
 }
 
+// a * b * s, one rounding to bf16
+__device__ __forceinline__ u32x4 mul_bf16x8_scaled(u32x4 a, u32x4 b, float s) {
+    u32x4 r;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) r[w] = pack_bf16(bf16_lo(a[w]) * bf16_lo(b[w]) * s, bf16_hi(a[w]) * bf16_hi(b[w]) * s);
+    return r;
+}
+
+// c + lo(x) + hi(x) for a packed pair of bf16 (v_dot2c_f32_bf16 against (1, 1))
+__device__ __forceinline__ float add_bf16x2(uint32_t x, float c) {
+    typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, x), __builtin_bit_cast(bf16x2_t, 0x3f803f80u), c, false);
+}
+
+__device__ __forceinline__ f32x16 splat16(float v) {
+    f32x16 r;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) r[i] = v;
+    return r;
+}
+
+// wave index as a scalar: branches on it are uniform and index arithmetic stays on the scalar unit
+__device__ __forceinline__ int wave_index() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
+
 __device__ __forceinline__ f32x16 mfma32(u32x4 a, u32x4 b, f32x16 c) {
     return __builtin_amdgcn_mfma_f32_32x32x16_bf16(as_bf16x8(a), as_bf16x8(b), c, 0, 0, 0);
 }

@@ -66,7 +66,7 @@ __global__ __launch_bounds__(512) void fwd8_kernel(KParams p) {
     const int hk = h / p.G;
 
     const int tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63;
+    const int wave = wave_index(), lane = tid & 63;
     const int c = lane & 31, hf = lane >> 5;
     const int i0 = tile * 32;
     const int i = i0 + c;
@@ -204,10 +204,9 @@ __global__ __launch_bounds__(512) void fwd8_kernel(KParams p) {
             u32x4 pb[2];
 #pragma unroll
             for (int rr = 0; rr < 16; rr += 2) {
-                float p0 = fast_exp2(X[rr]);
-                float p1 = fast_exp2(X[rr + 1]);
-                l += p0 + p1;
-                pb[rr >> 3][(rr & 7) >> 1] = pack_bf16(p0, p1);
+                const uint32_t pp = pack_bf16(fast_exp2(X[rr]), fast_exp2(X[rr + 1]));
+                l = add_bf16x2(pp, l);            // row sum of the rounded weights the MFMA consumes
+                pb[rr >> 3][(rr & 7) >> 1] = pp;
             }
 #pragma unroll
             for (int k2s = 0; k2s < 2; ++k2s)
