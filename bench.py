@@ -12,8 +12,10 @@ Algorithmic work (attended triples P per (batch, head), P = sum_i min(i+1,w1) mi
 `value` uses 18*D*B*H*P over the fwd+bwd time.  Each kernel is also timed on its own
 through the C ABI with HIP events on the launch stream; the `roofline` object is for
 the kernel with the longest launch, priced with the contractions that kernel needs
-for its own outputs (fwd 2: S, O; dQ/dK2/dV2 4: S, dP, G, T; dK1/dV1 4: S, dP, dK1, dV1;
-2*D flop each per triple).
+for its own outputs (fwd 2: S, O; dQ/dK2 pass 3: S, dP, G; dV2 pass 2: S, T; dK1 pass 3:
+S, dP, dK1; dV1 pass 2: S, dV1; 2*D flop each per triple).  The backward entry points
+that launch two passes are also timed whole (4 contractions each: what their outputs
+need when S and dP are shared).
 """
 import argparse
 import json
@@ -71,7 +73,7 @@ def main():
     ap.add_argument('--workload', default='cfg3_raw_kernel_b4_h8_n8192_d128_w512_w32', choices=sorted(WORKLOADS))
     ap.add_argument('--cpu-slices', type=int, default=4, help='(batch, head) slices of the CPU baseline sample (0 = skip)')
     ap.add_argument('--kernel-iters', type=int, default=5, help='launches per kernel for the per-kernel timing')
-    ap.add_argument('--only', default=None, help='time only this kernel through the C ABI (fwd, bwd_delta, bwd_dq_dkv2, bwd_dkv1); for profiling')
+    ap.add_argument('--only', default=None, help='time only this entry through the C ABI (fwd, bwd_delta, bwd_dq_dkv2, bwd_dkv1, bwd_dq_dk2_pass, bwd_dk1_pass, bwd_dv1_pass); for profiling')
     args = ap.parse_args()
     if args.gpus != 1:
         print('bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path exists)', file=sys.stderr)
@@ -150,13 +152,26 @@ def main():
                                                       arg(dv2), ws.data_ptr(), ws_bytes, sh)),
         'bwd_dkv1': (4, lambda: lib.sa2_bwd_dkv1(prob, *five, arg(dout), lse.data_ptr(), delta.data_ptr(), arg(dk1), arg(dv1), sh)),
     }
+    if w2 <= 32:
+        # the two-pass backward entry points, one pass (= one kernel) at a time
+        def one_pass(which, fn):
+            def run():
+                os.environ['SA2_BWD_PASS'] = which
+                try:
+                    return fn()
+                finally:
+                    del os.environ['SA2_BWD_PASS']
+            return run
+        launches['bwd_dq_dk2_pass'] = (3, one_pass('first', launches['bwd_dq_dkv2'][1]))
+        launches['bwd_dk1_pass'] = (3, one_pass('first', launches['bwd_dkv1'][1]))
+        launches['bwd_dv1_pass'] = (2, one_pass('second', launches['bwd_dkv1'][1]))
     kernels = {}
     if args.only is not None:
         # the later kernels read what the earlier ones wrote: run the chain once, untimed
-        for name, (_, fn) in launches.items():
+        for name in ('fwd', 'bwd_delta'):
             if name == args.only:
                 break
-            _native.check(fn())
+            _native.check(launches[name][1]())
         launches = {args.only: launches[args.only]}
     for name, (ncontr, fn) in launches.items():
         _native.check(fn())
@@ -176,9 +191,13 @@ def main():
         print(json.dumps({'workload': args.workload, 'kernels': kernels}))
         return
     hbm_bytes = {'fwd': 7 * B * N * H * D * 2 + 4 * B * H * N, 'bwd_delta': 3 * B * N * H * D * 2 + 4 * B * H * N}
-    dom = max((k for k in kernels if kernels[k]['contractions']), key=lambda k: kernels[k]['ms'])
+    # entries that are exactly one kernel launch (the two-pass entry points are timed per pass)
+    single = [k for k in kernels if kernels[k]['contractions'] and (w2 > 32 or k not in ('bwd_dq_dkv2', 'bwd_dkv1'))]
+    dom = max(single, key=lambda k: kernels[k]['ms'])
     achieved = kernels[dom]['tflops']
-    roofline = {'bound': 'mfma', 'kernel': dom, 'achieved': achieved, 'peak': PEAK_BF16_TFLOPS, 'unit': 'TFLOP/s',
+    symbols = {'fwd': 'sa2::fwd8_kernel<%d>' % D, 'bwd_dq_dk2_pass': 'sa2::bwd_q8_kernel<%d, true>' % D,
+               'bwd_dk1_pass': 'sa2::bwd_kv8_kernel<%d, true>' % D, 'bwd_dv1_pass': 'sa2::bwd_kv8_kernel<%d, false>' % D}
+    roofline = {'bound': 'mfma', 'kernel': dom, 'kernel_symbol': symbols.get(dom), 'achieved': achieved, 'peak': PEAK_BF16_TFLOPS, 'unit': 'TFLOP/s',
                 'frac': round(achieved / PEAK_BF16_TFLOPS, 4), 'traffic': None,
                 'launch_ms': kernels[dom]['ms'],
                 'flops_per_launch': kernels[dom]['contractions'] * unit}

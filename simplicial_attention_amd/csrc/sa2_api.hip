@@ -198,6 +198,16 @@ static int bwd_common(const sa2_problem *prob, const sa2_tensor *q, const sa2_te
     return SA2_OK;
 }
 
+// Profiling knob: SA2_BWD_PASS=first|second launches only one of the two passes of a
+// two-pass backward entry point (results are then incomplete); unset: both.
+static int bwd_pass_filter() {
+    const char *v = std::getenv("SA2_BWD_PASS");
+    if (!v) return 0;
+    if (std::strcmp(v, "first") == 0) return 1;
+    if (std::strcmp(v, "second") == 0) return 2;
+    return 0;
+}
+
 // rows of K2/V2 a 32-row query tile can reach: 32 own + (w2max - 1) below it
 static int qk2_w2max(int w2) { return w2 <= 32 ? 32 : 64; }
 
@@ -233,12 +243,13 @@ int sa2_bwd_dq_dkv2(const sa2_problem *prob, const sa2_tensor *q, const sa2_tens
     // SA2_BWD_QK2_IMPL=fused) take the fused four-wave kernel
     const char *impl = std::getenv("SA2_BWD_QK2_IMPL");
     const bool fused = w2max > 32 || (impl && std::strcmp(impl, "fused") == 0);
+    const int pass = bwd_pass_filter();
     if (!fused && prob->dim_head == 128) {
-        hipLaunchKernelGGL((sa2::bwd_q8_kernel<128, true>), dim3(grid), dim3(512), 0, s, k, ws);
-        hipLaunchKernelGGL((sa2::bwd_q8_kernel<128, false>), dim3(grid), dim3(512), 0, s, k, ws);
+        if (pass != 2) hipLaunchKernelGGL((sa2::bwd_q8_kernel<128, true>), dim3(grid), dim3(512), 0, s, k, ws);
+        if (pass != 1) hipLaunchKernelGGL((sa2::bwd_q8_kernel<128, false>), dim3(grid), dim3(512), 0, s, k, ws);
     } else if (!fused) {
-        hipLaunchKernelGGL((sa2::bwd_q8_kernel<64, true>), dim3(grid), dim3(512), 0, s, k, ws);
-        hipLaunchKernelGGL((sa2::bwd_q8_kernel<64, false>), dim3(grid), dim3(512), 0, s, k, ws);
+        if (pass != 2) hipLaunchKernelGGL((sa2::bwd_q8_kernel<64, true>), dim3(grid), dim3(512), 0, s, k, ws);
+        if (pass != 1) hipLaunchKernelGGL((sa2::bwd_q8_kernel<64, false>), dim3(grid), dim3(512), 0, s, k, ws);
     } else if (prob->dim_head == 128 && w2max == 32)
         hipLaunchKernelGGL((sa2::bwd_qk2_kernel<128, 32>), dim3(grid), dim3(256), 0, s, k, ws);
     else if (prob->dim_head == 128)
@@ -248,6 +259,7 @@ int sa2_bwd_dq_dkv2(const sa2_problem *prob, const sa2_tensor *q, const sa2_tens
     else
         hipLaunchKernelGGL((sa2::bwd_qk2_kernel<64, 64>), dim3(grid), dim3(256), 0, s, k, ws);
     SA2_TRY(after_launch("dq/dk2/dv2"));
+    if (!fused && pass == 1) return SA2_OK;    // profiling one pass: leave the reduction out of its timing
     const int64_t rows = (int64_t)prob->batch * prob->kv_heads * prob->seq_len;
     const int rows_per_block = 256 / (prob->dim_head / 8);
     const int cgrid = (int)((rows + rows_per_block - 1) / rows_per_block);
@@ -276,12 +288,13 @@ int sa2_bwd_dkv1(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor 
     // SA2_BWD_KV1_IMPL=fused) take the fused four-wave kernel
     const char *impl = std::getenv("SA2_BWD_KV1_IMPL");
     const bool fused = prob->w2 > 32 || (impl && std::strcmp(impl, "fused") == 0);
+    const int pass = bwd_pass_filter();
     if (!fused && prob->dim_head == 128) {
-        hipLaunchKernelGGL((sa2::bwd_kv8_kernel<128, true>), dim3(grid), dim3(512), 0, s, k);
-        hipLaunchKernelGGL((sa2::bwd_kv8_kernel<128, false>), dim3(grid), dim3(512), 0, s, k);
+        if (pass != 2) hipLaunchKernelGGL((sa2::bwd_kv8_kernel<128, true>), dim3(grid), dim3(512), 0, s, k);
+        if (pass != 1) hipLaunchKernelGGL((sa2::bwd_kv8_kernel<128, false>), dim3(grid), dim3(512), 0, s, k);
     } else if (!fused) {
-        hipLaunchKernelGGL((sa2::bwd_kv8_kernel<64, true>), dim3(grid), dim3(512), 0, s, k);
-        hipLaunchKernelGGL((sa2::bwd_kv8_kernel<64, false>), dim3(grid), dim3(512), 0, s, k);
+        if (pass != 2) hipLaunchKernelGGL((sa2::bwd_kv8_kernel<64, true>), dim3(grid), dim3(512), 0, s, k);
+        if (pass != 1) hipLaunchKernelGGL((sa2::bwd_kv8_kernel<64, false>), dim3(grid), dim3(512), 0, s, k);
     } else if (prob->dim_head == 128)
         hipLaunchKernelGGL(sa2::bwd_dkv1_kernel<128>, dim3(grid), dim3(256), 0, s, k);
     else
