@@ -145,10 +145,17 @@ def main():
     five = (arg(qd), arg(k1d), arg(k2d), arg(v1d), arg(v2d))
     ws_bytes = lib.sa2_bwd_workspace_bytes(prob)
     ws = torch.empty(ws_bytes, dtype=torch.uint8, device=dev)
+    # the forward's per-offset value partials, as the autograd Function keeps them
+    saved = t_save = m_save = None
+    from simplicial_attention_amd.two_simplicial_attention import save_partials_max_bytes
+    if w2 <= 32 and lib.sa2_saved_t_bytes(prob) <= save_partials_max_bytes():
+        t_save = torch.empty(lib.sa2_saved_t_bytes(prob), dtype=torch.uint8, device=dev)
+        m_save = torch.empty(lib.sa2_saved_m_bytes(prob), dtype=torch.uint8, device=dev)
+        saved = _native.saved_arg(t_save, m_save)
     launches = {
-        'fwd': (2, lambda: lib.sa2_fwd(prob, *five, arg(out), arg(res), lse.data_ptr(), sh)),
+        'fwd': (2, lambda: lib.sa2_fwd(prob, *five, arg(out), arg(res), lse.data_ptr(), saved, sh)),
         'bwd_delta': (0, lambda: lib.sa2_bwd_delta(prob, arg(out), arg(res), arg(dout), delta.data_ptr(), sh)),
-        'bwd_dq_dkv2': (4, lambda: lib.sa2_bwd_dq_dkv2(prob, *five, arg(dout), lse.data_ptr(), delta.data_ptr(), arg(dq), arg(dk2),
+        'bwd_dq_dkv2': (4, lambda: lib.sa2_bwd_dq_dkv2(prob, *five, arg(dout), lse.data_ptr(), delta.data_ptr(), saved, arg(dq), arg(dk2),
                                                       arg(dv2), ws.data_ptr(), ws_bytes, sh)),
         'bwd_dkv1': (4, lambda: lib.sa2_bwd_dkv1(prob, *five, arg(dout), lse.data_ptr(), delta.data_ptr(), arg(dk1), arg(dv1), sh)),
     }

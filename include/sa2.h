@@ -72,6 +72,22 @@ typedef struct sa2_tensor {
     int64_t stride_h;
 } sa2_tensor;
 
+/* Optional by-products of the forward that the backward can reuse instead of
+ * recomputing them (the reference keeps only q, k, v, out and lse for its backward,
+ * triton_two_simplicial_attention.py:800-805, and recomputes everything else):
+ *   t  bf16 [batch][heads][w2][seq_len][dim_head]:  T[b,h,d,i,:] = sum_j 2^(x_ij - m) v1[j,:]
+ *      for the offset d = i - k, x = scaled logit * log2(e)
+ *   m  fp32 [batch][heads][w2][seq_len]:            the reference m of that sum
+ * With them dV2[k] = sum_d dO[k+d] * T[d,k+d] * 2^(m - lse*log2e) needs no contraction
+ * in the backward.  Sizes: sa2_saved_t_bytes(), sa2_saved_m_bytes().  t 16-byte aligned. */
+typedef struct sa2_saved {
+    void  *t;
+    float *m;
+} sa2_saved;
+
+int64_t sa2_saved_t_bytes(const sa2_problem *prob);   /* -1 if the problem is invalid */
+int64_t sa2_saved_m_bytes(const sa2_problem *prob);
+
 /* Library version (SA2_VERSION of the build). */
 int sa2_version(void);
 
@@ -89,11 +105,13 @@ int sa2_supported(int32_t dim_head, int32_t w1, int32_t w2, int32_t dtype);
  * out_residual may be NULL; if given (same shape/dtype as out) it receives
  * bf16(out_fp32 - out), so that out + out_residual carries the fp32 accumulator to
  * about 16 mantissa bits.  The backward uses it to form delta without the rounding
- * error of the bf16 output (the reference forms delta from the rounded output, :282). */
+ * error of the bf16 output (the reference forms delta from the rounded output, :282).
+ * saved may be NULL; if given, its buffers are filled (see sa2_saved). */
 int sa2_fwd(const sa2_problem *prob,
             const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
             const sa2_tensor *v1, const sa2_tensor *v2,
-            const sa2_tensor *out, const sa2_tensor *out_residual, float *lse, void *hip_stream);
+            const sa2_tensor *out, const sa2_tensor *out_residual, float *lse,
+            const sa2_saved *saved, void *hip_stream);
 
 /* delta[b,h,n] = sum_d (out + out_residual) * dout; out_residual may be NULL.
  * Replaces backward_preprocess_do_o_dot
@@ -111,11 +129,13 @@ int64_t sa2_bwd_workspace_bytes(const sa2_problem *prob);
  * (triton_two_simplicial_attention.py:938-1004; kernel :515-712; dq :697-699,709;
  * dk2/dv2 :680-683, :695, :702-707).  One kernel owns the query rows (dQ complete,
  * dK2/dV2 as partial rows in the workspace), a second one sums the partial rows and
- * the query heads of a group.  No atomics; results are bitwise reproducible. */
+ * the query heads of a group.  No atomics; results are bitwise reproducible.
+ * saved may be NULL; if it holds what sa2_fwd wrote for these inputs (and w2 <= 32),
+ * dV2 is formed from it instead of from a recomputation of the attention weights. */
 int sa2_bwd_dq_dkv2(const sa2_problem *prob,
                     const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
                     const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *dout,
-                    const float *lse, const float *delta,
+                    const float *lse, const float *delta, const sa2_saved *saved,
                     const sa2_tensor *dq, const sa2_tensor *dk2, const sa2_tensor *dv2,
                     void *workspace, int64_t workspace_bytes, void *hip_stream);
 
@@ -130,14 +150,14 @@ int sa2_bwd_dkv1(const sa2_problem *prob,
 /* Whole backward: delta, dQ, dK1/dV1, dK2/dV2 in stream order.  Replaces the body
  * of SlidingTwoSimplicialAttention.backward (triton_two_simplicial_attention.py:808-1006).
  * delta_ws is a caller-owned fp32 (batch, heads, seq) buffer, workspace a caller-owned
- * buffer of at least sa2_bwd_workspace_bytes() bytes; out_residual may be NULL (see
- * sa2_fwd).  Gradients are
+ * buffer of at least sa2_bwd_workspace_bytes() bytes; out_residual and saved may be
+ * NULL (see sa2_fwd).  Gradients are
  * written in the activation dtype and need no prior zeroing. */
 int sa2_bwd(const sa2_problem *prob,
             const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
             const sa2_tensor *v1, const sa2_tensor *v2,
             const sa2_tensor *out, const sa2_tensor *out_residual, const sa2_tensor *dout,
-            const float *lse, float *delta_ws,
+            const float *lse, const sa2_saved *saved, float *delta_ws,
             const sa2_tensor *dq, const sa2_tensor *dk1, const sa2_tensor *dk2,
             const sa2_tensor *dv1, const sa2_tensor *dv2,
             void *workspace, int64_t workspace_bytes, void *hip_stream);

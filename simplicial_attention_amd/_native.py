@@ -24,8 +24,8 @@ STATUS_NAMES = {
     5: 'SA2_ERR_LAUNCH',
 }
 
-EXPORTS = ('sa2_version', 'sa2_last_error', 'sa2_supported', 'sa2_fwd', 'sa2_bwd_delta',
-           'sa2_bwd_workspace_bytes', 'sa2_bwd_dq_dkv2', 'sa2_bwd_dkv1', 'sa2_bwd')
+EXPORTS = ('sa2_version', 'sa2_last_error', 'sa2_supported', 'sa2_saved_t_bytes', 'sa2_saved_m_bytes', 'sa2_fwd',
+           'sa2_bwd_delta', 'sa2_bwd_workspace_bytes', 'sa2_bwd_dq_dkv2', 'sa2_bwd_dkv1', 'sa2_bwd')
 
 
 class Sa2Error(RuntimeError):
@@ -44,6 +44,11 @@ class Problem(ctypes.Structure):
 class TensorArg(ctypes.Structure):
     _fields_ = [('ptr', ctypes.c_void_p), ('stride_b', ctypes.c_int64), ('stride_n', ctypes.c_int64),
                 ('stride_h', ctypes.c_int64)]
+
+
+class Saved(ctypes.Structure):
+    """sa2_saved: optional forward by-products (per-offset T and its reference)."""
+    _fields_ = [('t', ctypes.c_void_p), ('m', ctypes.c_void_p)]
 
 
 _lib = None
@@ -69,6 +74,10 @@ def load() -> ctypes.CDLL:
                 '(or `python -c "import __graft_entry__ as g; g.build()"`)')
         lib = ctypes.CDLL(LIB_PATH)
         P, T, F, V = ctypes.POINTER(Problem), ctypes.POINTER(TensorArg), ctypes.c_void_p, ctypes.c_void_p
+        S = ctypes.POINTER(Saved)
+        for name in ('sa2_saved_t_bytes', 'sa2_saved_m_bytes'):
+            getattr(lib, name).restype = ctypes.c_int64
+            getattr(lib, name).argtypes = [P]
         lib.sa2_version.restype = ctypes.c_int
         lib.sa2_version.argtypes = []
         lib.sa2_last_error.restype = ctypes.c_char_p
@@ -76,17 +85,17 @@ def load() -> ctypes.CDLL:
         lib.sa2_supported.restype = ctypes.c_int
         lib.sa2_supported.argtypes = [ctypes.c_int32] * 4
         lib.sa2_fwd.restype = ctypes.c_int
-        lib.sa2_fwd.argtypes = [P, T, T, T, T, T, T, T, F, V]
+        lib.sa2_fwd.argtypes = [P, T, T, T, T, T, T, T, F, S, V]
         lib.sa2_bwd_delta.restype = ctypes.c_int
         lib.sa2_bwd_delta.argtypes = [P, T, T, T, F, V]
         lib.sa2_bwd_workspace_bytes.restype = ctypes.c_int64
         lib.sa2_bwd_workspace_bytes.argtypes = [P]
         lib.sa2_bwd_dq_dkv2.restype = ctypes.c_int
-        lib.sa2_bwd_dq_dkv2.argtypes = [P, T, T, T, T, T, T, F, F, T, T, T, V, ctypes.c_int64, V]
+        lib.sa2_bwd_dq_dkv2.argtypes = [P, T, T, T, T, T, T, F, F, S, T, T, T, V, ctypes.c_int64, V]
         lib.sa2_bwd_dkv1.restype = ctypes.c_int
         lib.sa2_bwd_dkv1.argtypes = [P, T, T, T, T, T, T, F, F, T, T, V]
         lib.sa2_bwd.restype = ctypes.c_int
-        lib.sa2_bwd.argtypes = [P, T, T, T, T, T, T, T, T, F, F, T, T, T, T, T, V, ctypes.c_int64, V]
+        lib.sa2_bwd.argtypes = [P, T, T, T, T, T, T, T, T, F, S, F, T, T, T, T, T, V, ctypes.c_int64, V]
         _lib = lib
         return lib
 
@@ -104,3 +113,8 @@ def tensor_arg(t) -> TensorArg:
 
 def problem(batch, seq_len, heads, kv_heads, dim_head, w1, w2, causal, scale) -> Problem:
     return Problem(batch, seq_len, heads, kv_heads, dim_head, int(w1), int(w2), int(bool(causal)), float(scale), SA2_BF16)
+
+
+def saved_arg(t, m) -> Saved:
+    """Device tensors for the forward's per-offset T (bf16) and reference (fp32) -> sa2_saved."""
+    return Saved(t.data_ptr(), m.data_ptr())

@@ -14,8 +14,7 @@
 #include "sa2_bwd_q8.hpp"
 #include "sa2_bwd_qk2.hpp"
 #include "sa2_common.hpp"
-#include "sa2_fwd.hpp"
-#include "sa2_fwd_ds.hpp"
+#include "sa2_lds.hpp"
 #include "sa2_fwd8.hpp"
 
 namespace {
@@ -105,9 +104,25 @@ int sa2_supported(int32_t dim_head, int32_t w1, int32_t w2, int32_t dtype) {
     return (dim_head == 64 || dim_head == 128) && w1 >= 1 && w2 >= 1 && w2 <= 64 && dtype == SA2_BF16;
 }
 
+static int check_saved(const sa2_saved *saved) {
+    if (!saved->t || !saved->m) return fail(SA2_ERR_NULL_POINTER, "saved->t or saved->m is NULL");
+    if ((reinterpret_cast<uintptr_t>(saved->t) & 15) != 0) return fail(SA2_ERR_ALIGNMENT, "saved->t must be 16-byte aligned");
+    return SA2_OK;
+}
+
+int64_t sa2_saved_t_bytes(const sa2_problem *prob) {
+    if (check_problem(prob) != SA2_OK) return -1;
+    return (int64_t)prob->batch * prob->heads * prob->w2 * prob->seq_len * prob->dim_head * 2;
+}
+
+int64_t sa2_saved_m_bytes(const sa2_problem *prob) {
+    if (check_problem(prob) != SA2_OK) return -1;
+    return (int64_t)prob->batch * prob->heads * prob->w2 * prob->seq_len * 4;
+}
+
 int sa2_fwd(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
             const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *out, const sa2_tensor *out_residual,
-            float *lse, void *hip_stream) {
+            float *lse, const sa2_saved *saved, void *hip_stream) {
     SA2_TRY(check_problem(prob));
     if (out_residual) SA2_TRY(check_tensor(out_residual, "out_residual"));
     SA2_TRY(check_tensor(q, "q"));
@@ -127,26 +142,16 @@ int sa2_fwd(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, 
     if (out_residual) k.o_lo = dev(out_residual);
     k.lse = lse;
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
-    const char *impl = std::getenv("SA2_FWD_IMPL");
-    if (impl && std::strcmp(impl, "chunk") == 0) {
-        int grid = prob->batch * prob->heads * ((prob->seq_len + 127) / 128);
-        if (prob->dim_head == 128)
-            hipLaunchKernelGGL(sa2::fwd_kernel<128>, dim3(grid), dim3(256), 0, s, k);
-        else
-            hipLaunchKernelGGL(sa2::fwd_kernel<64>, dim3(grid), dim3(256), 0, s, k);
-    } else if (impl && std::strcmp(impl, "ds") == 0) {
-        int grid = prob->batch * prob->heads * ((prob->seq_len + 31) / 32);
-        if (prob->dim_head == 128)
-            hipLaunchKernelGGL(sa2::fwd_ds_kernel<128>, dim3(grid), dim3(256), 0, s, k);
-        else
-            hipLaunchKernelGGL(sa2::fwd_ds_kernel<64>, dim3(grid), dim3(256), 0, s, k);
-    } else {
-        int grid = prob->batch * prob->heads * ((prob->seq_len + 31) / 32);
-        if (prob->dim_head == 128)
-            hipLaunchKernelGGL(sa2::fwd8_kernel<128>, dim3(grid), dim3(512), 0, s, k);
-        else
-            hipLaunchKernelGGL(sa2::fwd8_kernel<64>, dim3(grid), dim3(512), 0, s, k);
+    if (saved) {
+        SA2_TRY(check_saved(saved));
+        k.t_save = static_cast<char *>(saved->t);
+        k.m_save = saved->m;
     }
+    const int grid = prob->batch * prob->heads * ((prob->seq_len + 31) / 32);
+    if (prob->dim_head == 128)
+        hipLaunchKernelGGL(sa2::fwd8_kernel<128>, dim3(grid), dim3(512), 0, s, k);
+    else
+        hipLaunchKernelGGL(sa2::fwd8_kernel<64>, dim3(grid), dim3(512), 0, s, k);
     return after_launch("forward");
 }
 
@@ -219,8 +224,8 @@ int64_t sa2_bwd_workspace_bytes(const sa2_problem *prob) {
 
 int sa2_bwd_dq_dkv2(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
                     const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *dout, const float *lse,
-                    const float *delta, const sa2_tensor *dq, const sa2_tensor *dk2, const sa2_tensor *dv2,
-                    void *workspace, int64_t workspace_bytes, void *hip_stream) {
+                    const float *delta, const sa2_saved *saved, const sa2_tensor *dq, const sa2_tensor *dk2,
+                    const sa2_tensor *dv2, void *workspace, int64_t workspace_bytes, void *hip_stream) {
     sa2::KParams k;
     SA2_TRY(bwd_common(prob, q, k1, k2, v1, v2, dout, lse, delta, &k));
     SA2_TRY(check_tensor(dq, "dq"));
@@ -244,12 +249,20 @@ int sa2_bwd_dq_dkv2(const sa2_problem *prob, const sa2_tensor *q, const sa2_tens
     const char *impl = std::getenv("SA2_BWD_QK2_IMPL");
     const bool fused = w2max > 32 || (impl && std::strcmp(impl, "fused") == 0);
     const int pass = bwd_pass_filter();
+    // with the forward's saved per-offset T the dv2 pass (a recomputation of S and T) is
+    // replaced by a kernel that streams T once
+    const bool use_saved = saved != nullptr && !fused;
+    if (saved) {
+        SA2_TRY(check_saved(saved));
+        k.t_save = static_cast<char *>(saved->t);
+        k.m_save = saved->m;
+    }
     if (!fused && prob->dim_head == 128) {
         if (pass != 2) hipLaunchKernelGGL((sa2::bwd_q8_kernel<128, true>), dim3(grid), dim3(512), 0, s, k, ws);
-        if (pass != 1) hipLaunchKernelGGL((sa2::bwd_q8_kernel<128, false>), dim3(grid), dim3(512), 0, s, k, ws);
+        if (pass != 1 && !use_saved) hipLaunchKernelGGL((sa2::bwd_q8_kernel<128, false>), dim3(grid), dim3(512), 0, s, k, ws);
     } else if (!fused) {
         if (pass != 2) hipLaunchKernelGGL((sa2::bwd_q8_kernel<64, true>), dim3(grid), dim3(512), 0, s, k, ws);
-        if (pass != 1) hipLaunchKernelGGL((sa2::bwd_q8_kernel<64, false>), dim3(grid), dim3(512), 0, s, k, ws);
+        if (pass != 1 && !use_saved) hipLaunchKernelGGL((sa2::bwd_q8_kernel<64, false>), dim3(grid), dim3(512), 0, s, k, ws);
     } else if (prob->dim_head == 128 && w2max == 32)
         hipLaunchKernelGGL((sa2::bwd_qk2_kernel<128, 32>), dim3(grid), dim3(256), 0, s, k, ws);
     else if (prob->dim_head == 128)
@@ -259,14 +272,24 @@ int sa2_bwd_dq_dkv2(const sa2_problem *prob, const sa2_tensor *q, const sa2_tens
     else
         hipLaunchKernelGGL((sa2::bwd_qk2_kernel<64, 64>), dim3(grid), dim3(256), 0, s, k, ws);
     SA2_TRY(after_launch("dq/dk2/dv2"));
-    if (!fused && pass == 1) return SA2_OK;    // profiling one pass: leave the reduction out of its timing
+    if (!fused && pass == 1) return SA2_OK;    // profiling one pass: leave the reductions out of its timing
+    if (use_saved) {
+        const int rpb = 256 / (prob->dim_head / 8);
+        const int dgrid = prob->batch * prob->kv_heads * ((prob->seq_len + rpb - 1) / rpb);
+        if (prob->dim_head == 128)
+            hipLaunchKernelGGL(sa2::dv2_from_saved_kernel<128>, dim3(dgrid), dim3(256), 0, s, k);
+        else
+            hipLaunchKernelGGL(sa2::dv2_from_saved_kernel<64>, dim3(dgrid), dim3(256), 0, s, k);
+        SA2_TRY(after_launch("dv2 from saved partials"));
+    }
     const int64_t rows = (int64_t)prob->batch * prob->kv_heads * prob->seq_len;
     const int rows_per_block = 256 / (prob->dim_head / 8);
     const int cgrid = (int)((rows + rows_per_block - 1) / rows_per_block);
+    const int with_dv2 = use_saved ? 0 : 1;
     if (prob->dim_head == 128)
-        hipLaunchKernelGGL(sa2::dk2_dv2_combine_kernel<128>, dim3(cgrid), dim3(256), 0, s, k, ws, 31 + w2max);
+        hipLaunchKernelGGL(sa2::dk2_dv2_combine_kernel<128>, dim3(cgrid), dim3(256), 0, s, k, ws, 31 + w2max, with_dv2);
     else
-        hipLaunchKernelGGL(sa2::dk2_dv2_combine_kernel<64>, dim3(cgrid), dim3(256), 0, s, k, ws, 31 + w2max);
+        hipLaunchKernelGGL(sa2::dk2_dv2_combine_kernel<64>, dim3(cgrid), dim3(256), 0, s, k, ws, 31 + w2max, with_dv2);
     return after_launch("dk2/dv2 combine");
 }
 
@@ -304,12 +327,12 @@ int sa2_bwd_dkv1(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor 
 
 int sa2_bwd(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
             const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *out, const sa2_tensor *out_residual,
-            const sa2_tensor *dout, const float *lse, float *delta_ws, const sa2_tensor *dq, const sa2_tensor *dk1,
-            const sa2_tensor *dk2, const sa2_tensor *dv1, const sa2_tensor *dv2, void *workspace,
+            const sa2_tensor *dout, const float *lse, const sa2_saved *saved, float *delta_ws, const sa2_tensor *dq,
+            const sa2_tensor *dk1, const sa2_tensor *dk2, const sa2_tensor *dv1, const sa2_tensor *dv2, void *workspace,
             int64_t workspace_bytes, void *hip_stream) {
     SA2_TRY(sa2_bwd_delta(prob, out, out_residual, dout, delta_ws, hip_stream));
-    SA2_TRY(sa2_bwd_dq_dkv2(prob, q, k1, k2, v1, v2, dout, lse, delta_ws, dq, dk2, dv2, workspace, workspace_bytes,
-                            hip_stream));
+    SA2_TRY(sa2_bwd_dq_dkv2(prob, q, k1, k2, v1, v2, dout, lse, delta_ws, saved, dq, dk2, dv2, workspace,
+                            workspace_bytes, hip_stream));
     SA2_TRY(sa2_bwd_dkv1(prob, q, k1, k2, v1, v2, dout, lse, delta_ws, dk1, dv1, hip_stream));
     return SA2_OK;
 }

@@ -16,7 +16,7 @@
 #pragma once
 
 #include "sa2_common.hpp"
-#include "sa2_fwd_ds.hpp"
+#include "sa2_lds.hpp"
 
 namespace sa2 {
 

@@ -25,7 +25,7 @@
 #include <type_traits>
 
 #include "sa2_common.hpp"
-#include "sa2_fwd_ds.hpp"
+#include "sa2_lds.hpp"
 
 namespace sa2 {
 
@@ -370,6 +370,46 @@ __global__ __launch_bounds__(512) void bwd_q8_kernel(KParams p, float *ws) {
             *reinterpret_cast<float4 *>(wk + row * D + col) = *reinterpret_cast<const float4 *>(sc + row * C::SPITCH + col);
         }
     }
+}
+
+// dV2 from the forward's saved per-offset T:
+//     dv2[b,k,hk,:] = sum_g sum_dlt do[b,k+dlt,h,:] * T[b,h,dlt,k+dlt,:] * 2^(m[b,h,dlt,k+dlt] - lse2[b,h,k+dlt])
+// (h = hk*G + g).  Streams T once from HBM; a thread owns 8 d of one row k.
+template <int D>
+__global__ __launch_bounds__(256) void dv2_from_saved_kernel(KParams p) {
+    constexpr int LP = D / 8;                 // threads per row
+    constexpr int RPB = 256 / LP;             // rows per block
+    const int N = p.N;
+    const int nblk = (N + RPB - 1) / RPB;
+    const int blk = blockIdx.x % nblk;
+    const int bh = blockIdx.x / nblk;
+    const int hk = bh % p.HK, b = bh / p.HK;
+    const int k = blk * RPB + threadIdx.x / LP;
+    const int col = (threadIdx.x % LP) * 16;  // byte offset inside a row
+    if (k >= N) return;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const int nd = p.w2 < N - k ? p.w2 : N - k;
+    for (int g = 0; g < p.G; ++g) {
+        const int h = hk * p.G + g;
+        const int64_t bh_row = ((int64_t)b * p.H + h);
+        const char *dog = p.dout.ptr + b * p.dout.sb + h * p.dout.sh + col;
+        const float *lse = p.lse + bh_row * N;
+#pragma unroll 4
+        for (int dlt = 0; dlt < nd; ++dlt) {
+            const int i = k + dlt;
+            const int64_t srow = (bh_row * p.w2 + dlt) * N + i;
+            const u32x4 t = ld_global16(p.t_save + srow * (D * 2) + col);
+            const u32x4 o = ld_global16(dog + (int64_t)i * p.dout.sn);
+            const float w = fast_exp2(p.m_save[srow] - lse[i] * kLog2e);
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                acc[2 * x] += bf16_lo(o[x]) * bf16_lo(t[x]) * w;
+                acc[2 * x + 1] += bf16_hi(o[x]) * bf16_hi(t[x]) * w;
+            }
+        }
+    }
+    u32x4 r = {pack_bf16(acc[0], acc[1]), pack_bf16(acc[2], acc[3]), pack_bf16(acc[4], acc[5]), pack_bf16(acc[6], acc[7])};
+    st_global16(p.dv2.ptr + b * p.dv2.sb + (int64_t)k * p.dv2.sn + hk * p.dv2.sh + col, r);
 }
 
 }  // namespace sa2

@@ -22,7 +22,7 @@
 #include <type_traits>
 
 #include "sa2_common.hpp"
-#include "sa2_fwd_ds.hpp"
+#include "sa2_lds.hpp"
 
 namespace sa2 {
 
@@ -318,11 +318,12 @@ __global__ __launch_bounds__(256, 1) void bwd_qk2_kernel(KParams p, float *ws) {
     }
 }
 
-// dk2[b,k,hk,:] = scale * sum_g sum_tiles partial rows of k,  dv2 likewise (no scale).
+// dk2[b,k,hk,:] = scale * sum_g sum_tiles partial rows of k,  dv2 likewise (no scale;
+// left out if with_dv2 == 0: dv2 then comes from the forward's saved partials).
 // Workspace rows of a tile with first query row i0: index x <-> k = i0 - halo + x, so
 // rows 0..halo-1 are the halo below the tile and rows halo..halo+31 its own rows.
 template <int D>
-__global__ __launch_bounds__(256) void dk2_dv2_combine_kernel(KParams p, const float *ws, int srows) {
+__global__ __launch_bounds__(256) void dk2_dv2_combine_kernel(KParams p, const float *ws, int srows, int with_dv2) {
     constexpr int LP = D / 8;   // threads per row, 8 d each
     const int N = p.N, ntile = (N + 31) / 32;
     const int halo = srows - 32;
@@ -346,7 +347,7 @@ __global__ __launch_bounds__(256) void dk2_dv2_combine_kernel(KParams p, const f
 #pragma unroll
             for (int x = 0; x < 8; ++x) {
                 ak[x] += src[x];
-                av[x] += src[per_tensor + x];
+                if (with_dv2) av[x] += src[per_tensor + x];
             }
         }
     }
@@ -357,7 +358,7 @@ __global__ __launch_bounds__(256) void dk2_dv2_combine_kernel(KParams p, const f
         ov[w] = pack_bf16(av[2 * w], av[2 * w + 1]);
     }
     st_global16(p.dk2.ptr + b * p.dk2.sb + (int64_t)k * p.dk2.sn + hk * p.dk2.sh + piece * 16, ok);
-    st_global16(p.dv2.ptr + b * p.dv2.sb + (int64_t)k * p.dv2.sn + hk * p.dv2.sh + piece * 16, ov);
+    if (with_dv2) st_global16(p.dv2.ptr + b * p.dv2.sb + (int64_t)k * p.dv2.sn + hk * p.dv2.sh + piece * 16, ov);
 }
 
 }  // namespace sa2

@@ -34,6 +34,10 @@ struct KParams {
     DevTensor o_lo;       // optional bf16 residual out_fp32 - bf16(out); ptr == nullptr if absent
     float *lse;
     float *delta;
+    // optional by-products of the forward, reused by the backward (nullptr if absent):
+    // t_save bf16 [B][H][w2][N][D]: T = sum_j 2^(x_ij - m) v1_j per offset, m_save fp32 [B][H][w2][N]: m
+    char *t_save;
+    float *m_save;
     int B, N, H, HK, G;   // G = H / HK query heads per key/value head
     int w1, w2;
     float scale;          // softmax scale

@@ -11,8 +11,10 @@
 //     S^T = K1 A^T          A = q_i * k2_{i-dlt}   (bf16, built once per offset)
 //     P^T = exp2(S^T scale log2e - M_i)
 //     T^T += V1^T P^T       (V1 fragments through ds_read_b64_tr_b16)
-// Every wave keeps a private softmax reference M (fixed while an offset runs, see
-// sa2_fwd_ds.hpp) and row sum l.  The output accumulator is shared: an fp32 [32][D]
+// Every wave keeps a private softmax reference M and row sum l.  M stays fixed while an
+// offset runs (no per-tile rescale of T inside the hot loop); a tile whose logits leave the
+// safe exponent range [-32, 64] relative to M takes a slow path outside the loop that
+// moves M and rescales T and l.  The output accumulator is shared: an fp32 [32][D]
 // LDS buffer relative to a common reference Mc.  At the end of a round the waves
 // publish their references, agree on Mc = max, and add v2_{i-dlt} * T * 2^(M - Mc) in
 // eight barrier-separated phases; in phase ph wave w owns the d-slice (w + ph) mod 8,
@@ -23,7 +25,7 @@
 #include <type_traits>
 
 #include "sa2_common.hpp"
-#include "sa2_fwd_ds.hpp"
+#include "sa2_lds.hpp"
 
 namespace sa2 {
 
@@ -348,6 +350,23 @@ __global__ __launch_bounds__(512) void fwd8_kernel(KParams p) {
             for (int w = 0; w < 8; ++w) Mn = fmaxf(Mn, xm[w * 32 + c]);
             const float fo = (Mc == -INFINITY) ? 0.f : fast_exp2(Mc - Mn);   // rescale of the old content
             const float g = fresh ? 0.f : fast_exp2(M - Mn);                 // weight of this wave's T
+            // by-product for the backward: this offset's T and its reference
+            if (p.t_save && row_ok && dlt < p.w2) {
+                const int64_t srow_g = (((int64_t)b * p.H + h) * p.w2 + dlt) * N + i;
+                char *trow = p.t_save + srow_g * (D * 2) + 16 * hf * 2;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    u32x4 lo4, hi4;
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) {
+                        lo4[w] = pack_bf16(T[dt][2 * w], T[dt][2 * w + 1]);
+                        hi4[w] = pack_bf16(T[dt][8 + 2 * w], T[dt][8 + 2 * w + 1]);
+                    }
+                    st_global16(trow + dt * 64, lo4);
+                    st_global16(trow + dt * 64 + 16, hi4);
+                }
+                if (hf == 0) p.m_save[srow_g] = fresh ? 0.f : M;
+            }
             // re-centre the private reference on what this wave has seen
             if (!fresh) {
                 l *= fast_exp2(-seen);

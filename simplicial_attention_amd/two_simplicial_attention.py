@@ -8,6 +8,8 @@ by hand-written gfx950 kernels reached through the C ABI of libsa2.so.
 """
 from __future__ import annotations
 
+import os
+
 from functools import partial
 
 import torch
@@ -26,6 +28,13 @@ def _unit_inner_stride(t: Tensor) -> Tensor:
 
 def _stream_handle(device) -> int:
     return torch.cuda.current_stream(device).cuda_stream
+
+
+def save_partials_max_bytes() -> int:
+    """Largest per-call buffer of saved value partials the forward may allocate for the
+    backward (bytes).  ``SA2_SAVE_PARTIALS_MAX_GIB`` overrides the default of 16 GiB;
+    0 switches the saving off (the backward then recomputes, as the reference does)."""
+    return int(float(os.environ.get('SA2_SAVE_PARTIALS_MAX_GIB', '16')) * (1 << 30))
 
 
 class SlidingTwoSimplicialAttention(Function):
@@ -69,17 +78,25 @@ class SlidingTwoSimplicialAttention(Function):
         needs_grad = any(ctx.needs_input_grad[:5])
         residual = torch.empty_like(out) if needs_grad else None
         prob = _native.problem(batch, seq_len, heads, kv_heads, dim, w1, w2, True, scale)
+        # per-offset value partials T (and their references), kept for the backward when
+        # they fit the budget: dV2 then needs no recomputation of the attention weights
+        t_save = m_save = None
+        if needs_grad and w2 <= 32 and 0 < lib.sa2_saved_t_bytes(prob) <= save_partials_max_bytes():
+            t_save = torch.empty((batch, heads, w2, seq_len, dim), dtype=q.dtype, device=q.device)
+            m_save = torch.empty((batch, heads, w2, seq_len), dtype=torch.float32, device=q.device)
         with torch.cuda.device_of(q):
             _native.check(lib.sa2_fwd(prob, *(_native.tensor_arg(t) for t in (q, k1, k2, v1, v2, out)),
                                       _native.tensor_arg(residual) if needs_grad else None,
-                                      lse.data_ptr(), _stream_handle(q.device)))
-        ctx.save_for_backward(q, k1, k2, v1, v2, out, lse, residual)
+                                      lse.data_ptr(),
+                                      _native.saved_arg(t_save, m_save) if t_save is not None else None,
+                                      _stream_handle(q.device)))
+        ctx.save_for_backward(q, k1, k2, v1, v2, out, lse, residual, t_save, m_save)
         ctx.problem = (batch, seq_len, heads, kv_heads, dim, w1, w2, scale)
         return out
 
     @staticmethod
     def backward(ctx, dout):
-        q, k1, k2, v1, v2, out, lse, residual = ctx.saved_tensors
+        q, k1, k2, v1, v2, out, lse, residual, t_save, m_save = ctx.saved_tensors
         batch, seq_len, heads, kv_heads, dim, w1, w2, scale = ctx.problem
         dout = _unit_inner_stride(dout)
         lib = _native.load()
@@ -93,7 +110,9 @@ class SlidingTwoSimplicialAttention(Function):
         with torch.cuda.device_of(q):
             _native.check(lib.sa2_bwd(prob, arg(q), arg(k1), arg(k2), arg(v1), arg(v2), arg(out),
                                       arg(residual) if residual is not None else None, arg(dout),
-                                      lse.data_ptr(), delta.data_ptr(),
+                                      lse.data_ptr(),
+                                      _native.saved_arg(t_save, m_save) if t_save is not None else None,
+                                      delta.data_ptr(),
                                       arg(dq), arg(dk1), arg(dk2), arg(dv1), arg(dv2),
                                       workspace.data_ptr(), ws_bytes, _stream_handle(q.device)))
         return dq, dk1, dk2, dv1, dv2, None, None, None

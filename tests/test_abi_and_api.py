@@ -55,7 +55,7 @@ def test_argument_validation_happens_before_any_launch(lib):
     lse = ctypes.c_void_p(0x2000)
 
     def fwd(prob, *tensors, lse_ptr=lse):
-        return lib.sa2_fwd(prob, *tensors, None, lse_ptr, None)
+        return lib.sa2_fwd(prob, *tensors, None, lse_ptr, None, None)
 
     assert fwd(None, t, t, t, t, t, t) == 1
     assert fwd(good, None, t, t, t, t, t) == 1
@@ -77,12 +77,18 @@ def test_argument_validation_happens_before_any_launch(lib):
     need = lib.sa2_bwd_workspace_bytes(good)
     assert need == 2 * 1 * 2 * 2 * 63 * 128 * 4          # 2 tensors, B*H*tiles blocks of 63 fp32 rows
     assert lib.sa2_bwd_workspace_bytes(None) == -1
-    assert lib.sa2_bwd_dq_dkv2(good, t, t, t, t, t, t, None, lse, t, t, t, lse, need, None) == 1
-    assert lib.sa2_bwd_dq_dkv2(good, t, t, t, t, t, t, lse, lse, t, t, t, None, need, None) == 1
-    assert lib.sa2_bwd_dq_dkv2(good, t, t, t, t, t, t, lse, lse, t, t, t, lse, need - 1, None) == 2
-    assert lib.sa2_bwd_dq_dkv2(good, t, t, t, t, t, t, lse, lse, t, t, _dummy(ptr=0x1004), lse, need, None) == 4
+    assert lib.sa2_bwd_dq_dkv2(good, t, t, t, t, t, t, None, lse, None, t, t, t, lse, need, None) == 1
+    assert lib.sa2_bwd_dq_dkv2(good, t, t, t, t, t, t, lse, lse, None, t, t, t, None, need, None) == 1
+    assert lib.sa2_bwd_dq_dkv2(good, t, t, t, t, t, t, lse, lse, None, t, t, t, lse, need - 1, None) == 2
+    assert lib.sa2_bwd_dq_dkv2(good, t, t, t, t, t, t, lse, lse, None, t, t, _dummy(ptr=0x1004), lse, need, None) == 4
     assert lib.sa2_bwd_dkv1(good, t, t, t, t, t, t, lse, lse, None, t, None) == 1
-    assert lib.sa2_bwd(good, t, t, t, t, t, None, None, t, lse, lse, t, t, t, t, t, lse, need, None) == 1
+    assert lib.sa2_bwd(good, t, t, t, t, t, None, None, t, lse, None, lse, t, t, t, t, t, lse, need, None) == 1
+    # saved forward partials: sizes, and NULL members are refused
+    assert lib.sa2_saved_t_bytes(good) == 1 * 2 * 32 * 64 * 128 * 2
+    assert lib.sa2_saved_m_bytes(good) == 1 * 2 * 32 * 64 * 4
+    assert lib.sa2_saved_t_bytes(None) == -1
+    assert lib.sa2_fwd(good, t, t, t, t, t, t, None, lse, ctypes.byref(_native.Saved(None, None)), None) == 1
+    assert lib.sa2_fwd(good, t, t, t, t, t, t, None, lse, ctypes.byref(_native.Saved(0x1004, 0x2000)), None) == 4
 
 
 def test_function_rejects_what_the_kernels_do_not_cover():

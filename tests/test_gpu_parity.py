@@ -82,12 +82,24 @@ def test_lse_matches_oracle():
     lse = torch.empty(b, h, n, dtype=torch.float32, device='cuda')
     lib = _native.load()
     prob = _native.problem(b, n, h, h, d, w1, w2, True, d ** -0.5)
-    _native.check(lib.sa2_fwd(prob, *(_native.tensor_arg(t) for t in (*ts, out)), None, lse.data_ptr(),
+    _native.check(lib.sa2_fwd(prob, *(_native.tensor_arg(t) for t in (*ts, out)), None, lse.data_ptr(), None,
                               torch.cuda.current_stream().cuda_stream))
     torch.cuda.synchronize()
     from oracle import reference_attend as R
     _, ref = R.windowed_banded(*[t.float() for t in (q, k1, k2, v1, v2)], w1, w2)
     assert torch.allclose(lse.cpu(), ref, atol=2e-2, rtol=1e-2)
+
+
+@pytest.mark.parametrize('shape', [(2, 320, 4, 2, 128, 96, 16), (1, 200, 2, 2, 64, 64, 32)])
+def test_backward_that_recomputes_instead_of_using_saved_partials(shape, monkeypatch):
+    """SA2_SAVE_PARTIALS_MAX_GIB=0: the forward keeps no per-offset T and dV2 comes from
+    the recomputing pass (what the reference does)."""
+    monkeypatch.setenv('SA2_SAVE_PARTIALS_MAX_GIB', '0')
+    b, n, hq, hk, d, w1, w2 = shape
+    ins = U.make_inputs(b, n, hq, hk, d, seed=23, std=d ** -0.5)
+    ref_out, _, ref_grads = U.oracle_fwd_bwd(*ins, w1, w2)
+    out, grads = U.hip_fwd_bwd(*ins, w1, w2)
+    U.check_all(out, grads, ref_out, ref_grads)
 
 
 def test_backward_is_deterministic():
