@@ -73,7 +73,7 @@ def main():
     ap.add_argument('--workload', default='cfg3_raw_kernel_b4_h8_n8192_d128_w512_w32', choices=sorted(WORKLOADS))
     ap.add_argument('--cpu-slices', type=int, default=4, help='(batch, head) slices of the CPU baseline sample (0 = skip)')
     ap.add_argument('--kernel-iters', type=int, default=5, help='launches per kernel for the per-kernel timing')
-    ap.add_argument('--only', default=None, help='time only this entry through the C ABI (fwd, bwd_delta, bwd_dq_dkv2, bwd_dkv1, bwd_dq_dk2_pass, bwd_dk1_pass, bwd_dv1_pass); for profiling')
+    ap.add_argument('--only', default=None, help='time only this entry through the C ABI (fwd, bwd_delta, bwd_dq_dkv2, bwd_dkv1, bwd_dq_dk2_pass, bwd_dk1_pass, bwd_dv1_pass), or `copy`: a 1 GiB device copy that calibrates HBM counters; for profiling')
     args = ap.parse_args()
     if args.gpus != 1:
         print('bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path exists)', file=sys.stderr)
@@ -91,6 +91,15 @@ def main():
 
     B, H, HK, N, D, w1, w2 = WORKLOADS[args.workload]
     dev = torch.device('cuda:0')
+    if args.only == 'copy':
+        # plain device copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters
+        src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)
+        dst = torch.empty_like(src)
+        for _ in range(args.kernel_iters):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({'copy_bytes_read': 1 << 30, 'copy_bytes_written': 1 << 30, 'launches': args.kernel_iters}))
+        return
     g = torch.Generator(device='cpu').manual_seed(2)
     mk = lambda h, s: (torch.randn(B, N, h, D, generator=g) * s).bfloat16().to(dev)
     q = mk(H, D ** -0.5)
@@ -204,8 +213,15 @@ def main():
     achieved = kernels[dom]['tflops']
     symbols = {'fwd': 'sa2::fwd8_kernel<%d>' % D, 'bwd_dq_dk2_pass': 'sa2::bwd_q8_kernel<%d, true>' % D,
                'bwd_dk1_pass': 'sa2::bwd_kv8_kernel<%d, true>' % D, 'bwd_dv1_pass': 'sa2::bwd_kv8_kernel<%d, false>' % D}
+    # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `--only <entry>` on this
+    # workload, scaled by what the same counters read for a 1 GiB device copy (profiles/pmc_cfg3_mfma_kernels.txt)
+    measured_traffic = {
+        'cfg3_raw_kernel_b4_h8_n8192_d128_w512_w32': {
+            'fwd': 2687567016, 'bwd_dq_dk2_pass': 742447594, 'bwd_dk1_pass': 1222089896, 'bwd_dv1_pass': 517111401},
+    }
+    traffic = measured_traffic.get(args.workload, {}).get(dom)
     roofline = {'bound': 'mfma', 'kernel': dom, 'kernel_symbol': symbols.get(dom), 'achieved': achieved, 'peak': PEAK_BF16_TFLOPS, 'unit': 'TFLOP/s',
-                'frac': round(achieved / PEAK_BF16_TFLOPS, 4), 'traffic': None,
+                'frac': round(achieved / PEAK_BF16_TFLOPS, 4), 'traffic': traffic,
                 'launch_ms': kernels[dom]['ms'],
                 'flops_per_launch': kernels[dom]['contractions'] * unit}
 

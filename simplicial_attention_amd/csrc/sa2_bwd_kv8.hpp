@@ -191,18 +191,45 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
         const int dlt = 2 * s.m + sub;
         const bool dead = dlt > dmax_of(s.it);        // odd number of offsets: the last pair is half empty
         const int dl = dead ? 0 : dlt;
+        // all LDS reads of a product first, then the multiplies and the writes: the read
+        // latency is paid once per product, not once per piece
+        u32x4 fq[L::LPT], fk[L::LPT];
+        int row[L::LPT], col[L::LPT];
 #pragma unroll
         for (int x = 0; x < L::LPT; ++x) {
             const int pc = x * 256 + t8;
-            const int row = pc / PPR, col = (pc % PPR) * 16;
-            const int krow = row - dl + L::HALO;
-            const u32x4 a = mul_bf16x8(ld_lds16(lds + L::QS + row * L::RP + col), ld_lds16(lds + L::K2S + krow * L::RP + col));
-            *reinterpret_cast<u32x4 *>(stage + L::AS + row * PITCH + col) = a;
-            if constexpr (DK) *reinterpret_cast<u32x4 *>(stage + L::TR + row * L::TPITCH + col) = a;
-            __builtin_amdgcn_sched_barrier(0);        // one product at a time: keeps the build's registers few
-            const u32x4 bb = mul_bf16x8(ld_lds16(lds + L::DOS + row * L::RP + col), ld_lds16(lds + L::V2S + krow * L::RP + col));
-            *reinterpret_cast<u32x4 *>(stage + (DK ? L::BS + row * PITCH : L::TR + row * L::TPITCH) + col) = bb;
+            row[x] = pc / PPR;
+            col[x] = (pc % PPR) * 16;
+            fq[x] = ld_lds16(lds + L::QS + row[x] * L::RP + col[x]);
+            fk[x] = ld_lds16(lds + L::K2S + (row[x] - dl + L::HALO) * L::RP + col[x]);
+        }
+        u32x4 fo[L::LPT], fv[L::LPT];
+        if constexpr (DK) __builtin_amdgcn_sched_barrier(0);   // the dk1 pass has no registers for both products at once
+#pragma unroll
+        for (int x = 0; x < L::LPT; ++x) {
+            if constexpr (!DK) {
+                fo[x] = ld_lds16(lds + L::DOS + row[x] * L::RP + col[x]);
+                fv[x] = ld_lds16(lds + L::V2S + (row[x] - dl + L::HALO) * L::RP + col[x]);
+            }
+        }
+#pragma unroll
+        for (int x = 0; x < L::LPT; ++x) {
+            const u32x4 a = mul_bf16x8(fq[x], fk[x]);
+            *reinterpret_cast<u32x4 *>(stage + L::AS + row[x] * PITCH + col[x]) = a;
+            if constexpr (DK) *reinterpret_cast<u32x4 *>(stage + L::TR + row[x] * L::TPITCH + col[x]) = a;
+        }
+        if constexpr (DK) {
             __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int x = 0; x < L::LPT; ++x) {
+                fo[x] = ld_lds16(lds + L::DOS + row[x] * L::RP + col[x]);
+                fv[x] = ld_lds16(lds + L::V2S + (row[x] - dl + L::HALO) * L::RP + col[x]);
+            }
+        }
+#pragma unroll
+        for (int x = 0; x < L::LPT; ++x) {
+            const u32x4 bb = mul_bf16x8(fo[x], fv[x]);
+            *reinterpret_cast<u32x4 *>(stage + (DK ? L::BS + row[x] * PITCH : L::TR + row[x] * L::TPITCH) + col[x]) = bb;
         }
         if (t8 < 32) {
             const int i = 32 * s.it + t8;
