@@ -244,10 +244,12 @@ __global__ __launch_bounds__(512) void bwd_q8_kernel(KParams p, float *ws) {
 #pragma unroll
             for (int rr = 0; rr < 16; ++rr) X[rr] = X[rr] * c2 - lse2;
             if constexpr (MASKED) {
+                // row j = 32 t + 4 hf + e (e = 8 (rr / 4) + rr % 4) is attended iff 0 <= i - j < w1;
+                // lanes without a valid k2 row get a distance no e can bring into range
+                const int rel = col_ok ? i - 32 * t - 4 * hf : -(1 << 30);
 #pragma unroll
                 for (int rr = 0; rr < 16; ++rr) {
-                    int j = 32 * t + 8 * (rr >> 2) + 4 * hf + (rr & 3);
-                    bool ok = col_ok && (j <= i) && (j + p.w1 > i);
+                    const bool ok = (unsigned)(rel - (8 * (rr >> 2) + (rr & 3))) < (unsigned)p.w1;
                     X[rr] = ok ? X[rr] : -INFINITY;
                 }
             }
