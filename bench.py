@@ -73,7 +73,7 @@ def main():
     ap.add_argument('--workload', default='cfg3_raw_kernel_b4_h8_n8192_d128_w512_w32', choices=sorted(WORKLOADS))
     ap.add_argument('--cpu-slices', type=int, default=4, help='(batch, head) slices of the CPU baseline sample (0 = skip)')
     ap.add_argument('--kernel-iters', type=int, default=5, help='launches per kernel for the per-kernel timing')
-    ap.add_argument('--only', default=None, help='time only this entry through the C ABI (fwd, bwd_delta, bwd_dq_dkv2, bwd_dkv1, bwd_dq_dk2_pass, bwd_dk1_pass, bwd_dv1_pass), or `copy`: a 1 GiB device copy that calibrates HBM counters; for profiling')
+    ap.add_argument('--only', default=None, help='time only this entry through the C ABI (fwd, bwd_delta, bwd_dq_dkv2, bwd_dkv1, bwd_dq_dk2_pass, bwd_dk1_pass, bwd_dv1_pass), `copy`: a 1 GiB device copy that calibrates HBM counters; `module_cfg2`: the module forward of config 2 and the fused qkv-norm kernel; for profiling')
     args = ap.parse_args()
     if args.gpus != 1:
         print('bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path exists)', file=sys.stderr)
@@ -91,6 +91,40 @@ def main():
 
     B, H, HK, N, D, w1, w2 = WORKLOADS[args.workload]
     dev = torch.device('cuda:0')
+    if args.only == 'module_cfg2':
+        # BASELINE config 2: the multi-head module, tokens (2, 1024, 512), dim_head 64, 8 heads, forward,
+        # with and without the fused split + RMSNorm kernel; and that kernel alone at the config-3 token count
+        from simplicial_attention_amd import SlidingWindowTwoSimplicialMHA
+        from simplicial_attention_amd.qkv_norm import FusedQKVNorm
+        torch.manual_seed(1)
+        m = SlidingWindowTwoSimplicialMHA(512, dim_head=64, heads=8, w1=512, w2=32).bfloat16().to(dev)
+        tokens = torch.randn(2, 1024, 512, device=dev).bfloat16()
+
+        def timed(fn, iters=50):
+            for _ in range(5):
+                fn()
+            torch.cuda.synchronize()
+            a, b_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record()
+            for _ in range(iters):
+                fn()
+            b_.record()
+            torch.cuda.synchronize()
+            return a.elapsed_time(b_) / iters
+        res = {}
+        with torch.no_grad():
+            for fused in (True, False):
+                m.fused_qkv_norm = fused
+                res['module_fwd_ms_fused' if fused else 'module_fwd_ms_unfused'] = round(timed(lambda: m(tokens)), 4)
+            bq, nq, hq, dq_ = 4, 8192, 8, 128
+            qkv = torch.randn(bq, nq, 5 * hq * dq_, device=dev).bfloat16()
+            w = torch.ones(dq_, device=dev).bfloat16()
+            ms = timed(lambda: FusedQKVNorm.apply(qkv, w, w, w, w, w, hq, hq, dq_, 1e-6), 20)
+            nbytes = 2 * qkv.numel() * 2 + 4 * bq * nq * 5 * hq
+            res['qkv_norm_fwd'] = {'tokens': bq * nq, 'channels': 5 * hq * dq_, 'ms': round(ms, 4),
+                                   'hbm_bytes': nbytes, 'achieved_gbs': round(nbytes / ms / 1e6, 1), 'peak_gbs': PEAK_HBM_GBS}
+        print(json.dumps(res))
+        return
     if args.only == 'copy':
         # plain device copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters
         src = torch.empty(1 << 30, dtype=torch.uint8, device=dev).fill_(1)

@@ -162,6 +162,36 @@ int sa2_bwd(const sa2_problem *prob,
             const sa2_tensor *dv1, const sa2_tensor *dv2,
             void *workspace, int64_t workspace_bytes, void *hip_stream);
 
+/* ---- module pre-processing around the attention core (first of the "next" rows) ----
+ *
+ * Fused split + per-head RMSNorm of the qkv projection.  Replaces, for
+ * number_key_value_sets = 2 and head_first_dim = False, the split / unflatten / chunk /
+ * five RMSNorm calls of HigherOrderAttention.forward (simplicial_mha.py:116-127): reads
+ * the projection output qkv[b, n, :] (bf16, channels q (head, d) | k (head, set, d) |
+ * v (head, set, d), row_stride elements between tokens) once and writes the five
+ * (batch, seq, heads, dim_head) tensors the attention entry points take.
+ * w_* are bf16 [dim_head] RMSNorm weights (NULL: ones); y = x * rsqrt(mean(x^2) + eps) * w
+ * in fp32, rounded once.  rstd (fp32 [batch*seq][heads + 4*kv_heads]) is kept for the
+ * backward.  prob->w1/w2/scale are not used. */
+int sa2_qkv_norm_fwd(const sa2_problem *prob, const void *qkv, int64_t row_stride,
+                     const void *w_q, const void *w_k1, const void *w_k2, const void *w_v1, const void *w_v2,
+                     float eps,
+                     const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
+                     const sa2_tensor *v1, const sa2_tensor *v2, float *rstd, void *hip_stream);
+
+/* Bytes of workspace sa2_qkv_norm_bwd needs (partial weight gradients); -1 if invalid. */
+int64_t sa2_qkv_norm_bwd_workspace_bytes(const sa2_problem *prob);
+
+/* Backward of sa2_qkv_norm_fwd: dqkv (bf16, layout of qkv) from the gradients of the five
+ * outputs, and dw (fp32 [5][dim_head], order q, k1, k2, v1, v2; written, not accumulated).
+ * The autograd of the reference's five RMSNorm modules plus the backward of split /
+ * chunk (simplicial_mha.py:116-127).  Bitwise reproducible (no atomics). */
+int sa2_qkv_norm_bwd(const sa2_problem *prob, const void *qkv, int64_t row_stride,
+                     const void *w_q, const void *w_k1, const void *w_k2, const void *w_v1, const void *w_v2,
+                     const sa2_tensor *dq, const sa2_tensor *dk1, const sa2_tensor *dk2,
+                     const sa2_tensor *dv1, const sa2_tensor *dv2, const float *rstd,
+                     void *dqkv, float *dw, void *workspace, int64_t workspace_bytes, void *hip_stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -25,7 +25,8 @@ STATUS_NAMES = {
 }
 
 EXPORTS = ('sa2_version', 'sa2_last_error', 'sa2_supported', 'sa2_saved_t_bytes', 'sa2_saved_m_bytes', 'sa2_fwd',
-           'sa2_bwd_delta', 'sa2_bwd_workspace_bytes', 'sa2_bwd_dq_dkv2', 'sa2_bwd_dkv1', 'sa2_bwd')
+           'sa2_bwd_delta', 'sa2_bwd_workspace_bytes', 'sa2_bwd_dq_dkv2', 'sa2_bwd_dkv1', 'sa2_bwd',
+           'sa2_qkv_norm_fwd', 'sa2_qkv_norm_bwd_workspace_bytes', 'sa2_qkv_norm_bwd')
 
 
 class Sa2Error(RuntimeError):
@@ -96,6 +97,13 @@ def load() -> ctypes.CDLL:
         lib.sa2_bwd_dkv1.argtypes = [P, T, T, T, T, T, T, F, F, T, T, V]
         lib.sa2_bwd.restype = ctypes.c_int
         lib.sa2_bwd.argtypes = [P, T, T, T, T, T, T, T, T, F, S, F, T, T, T, T, T, V, ctypes.c_int64, V]
+        I64 = ctypes.c_int64
+        lib.sa2_qkv_norm_fwd.restype = ctypes.c_int
+        lib.sa2_qkv_norm_fwd.argtypes = [P, V, I64, V, V, V, V, V, ctypes.c_float, T, T, T, T, T, F, V]
+        lib.sa2_qkv_norm_bwd_workspace_bytes.restype = I64
+        lib.sa2_qkv_norm_bwd_workspace_bytes.argtypes = [P]
+        lib.sa2_qkv_norm_bwd.restype = ctypes.c_int
+        lib.sa2_qkv_norm_bwd.argtypes = [P, V, I64, V, V, V, V, V, T, T, T, T, T, F, V, F, V, I64, V]
         _lib = lib
         return lib
 

@@ -15,6 +15,7 @@
 #include "sa2_bwd_qk2.hpp"
 #include "sa2_common.hpp"
 #include "sa2_lds.hpp"
+#include "sa2_qkv_norm.hpp"
 #include "sa2_fwd8.hpp"
 
 namespace {
@@ -335,6 +336,97 @@ int sa2_bwd(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, 
                             workspace_bytes, hip_stream));
     SA2_TRY(sa2_bwd_dkv1(prob, q, k1, k2, v1, v2, dout, lse, delta_ws, dk1, dv1, hip_stream));
     return SA2_OK;
+}
+
+// ---- fused split + per-head RMSNorm of the qkv projection -------------------------------
+static constexpr int kNormMaxBlocks = 2048;
+
+static int norm_groups(const sa2_problem *prob) {
+    const int64_t rows = (int64_t)prob->batch * prob->seq_len * (prob->heads + 4 * prob->kv_heads);
+    const int rpb = 256 / (prob->dim_head / 8);
+    return (int)((rows + rpb - 1) / rpb);
+}
+
+static int norm_common(const sa2_problem *prob, const void *qkv, int64_t row_stride, const sa2_tensor *const t[5],
+                       const void *const w[5], const float *rstd, sa2::NormParams *np) {
+    SA2_TRY(check_problem(prob));
+    if (!qkv) return fail(SA2_ERR_NULL_POINTER, "qkv is NULL");
+    if (!rstd) return fail(SA2_ERR_NULL_POINTER, "rstd is NULL");
+    const int64_t channels = (int64_t)(prob->heads + 4 * prob->kv_heads) * prob->dim_head;
+    if (row_stride < channels) return fail(SA2_ERR_BAD_SHAPE, "row_stride %lld is smaller than the %lld channels of a token",
+                                           (long long)row_stride, (long long)channels);
+    if ((reinterpret_cast<uintptr_t>(qkv) & 15) != 0 || row_stride % 8 != 0)
+        return fail(SA2_ERR_ALIGNMENT, "qkv rows must be 16-byte aligned");
+    static const char *names[5] = {"q", "k1", "k2", "v1", "v2"};
+    *np = sa2::NormParams{};
+    for (int x = 0; x < 5; ++x) {
+        SA2_TRY(check_tensor(t[x], names[x]));
+        np->t[x] = dev(t[x]);
+        if (w[x] && (reinterpret_cast<uintptr_t>(w[x]) & 15) != 0) return fail(SA2_ERR_ALIGNMENT, "norm weights must be 16-byte aligned");
+        np->w[x] = static_cast<const char *>(w[x]);
+    }
+    np->qkv = static_cast<const char *>(qkv);
+    np->row_stride = row_stride * 2;
+    np->rstd = const_cast<float *>(rstd);
+    np->B = prob->batch;
+    np->N = prob->seq_len;
+    np->H = prob->heads;
+    np->HK = prob->kv_heads;
+    return SA2_OK;
+}
+
+int sa2_qkv_norm_fwd(const sa2_problem *prob, const void *qkv, int64_t row_stride, const void *w_q, const void *w_k1,
+                     const void *w_k2, const void *w_v1, const void *w_v2, float eps, const sa2_tensor *q,
+                     const sa2_tensor *k1, const sa2_tensor *k2, const sa2_tensor *v1, const sa2_tensor *v2, float *rstd,
+                     void *hip_stream) {
+    const sa2_tensor *const t[5] = {q, k1, k2, v1, v2};
+    const void *const w[5] = {w_q, w_k1, w_k2, w_v1, w_v2};
+    sa2::NormParams np;
+    SA2_TRY(norm_common(prob, qkv, row_stride, t, w, rstd, &np));
+    np.eps = eps;
+    hipStream_t s = static_cast<hipStream_t>(hip_stream);
+    const int grid = norm_groups(prob);
+    if (prob->dim_head == 128)
+        hipLaunchKernelGGL(sa2::qkv_norm_fwd_kernel<128>, dim3(grid), dim3(256), 0, s, np);
+    else
+        hipLaunchKernelGGL(sa2::qkv_norm_fwd_kernel<64>, dim3(grid), dim3(256), 0, s, np);
+    return after_launch("qkv norm forward");
+}
+
+int64_t sa2_qkv_norm_bwd_workspace_bytes(const sa2_problem *prob) {
+    if (check_problem(prob) != SA2_OK) return -1;
+    const int groups = norm_groups(prob);
+    const int blocks = groups < kNormMaxBlocks ? groups : kNormMaxBlocks;
+    return (int64_t)blocks * 5 * prob->dim_head * 4;
+}
+
+int sa2_qkv_norm_bwd(const sa2_problem *prob, const void *qkv, int64_t row_stride, const void *w_q, const void *w_k1,
+                     const void *w_k2, const void *w_v1, const void *w_v2, const sa2_tensor *dq, const sa2_tensor *dk1,
+                     const sa2_tensor *dk2, const sa2_tensor *dv1, const sa2_tensor *dv2, const float *rstd, void *dqkv,
+                     float *dw, void *workspace, int64_t workspace_bytes, void *hip_stream) {
+    const sa2_tensor *const t[5] = {dq, dk1, dk2, dv1, dv2};
+    const void *const w[5] = {w_q, w_k1, w_k2, w_v1, w_v2};
+    sa2::NormParams np;
+    SA2_TRY(norm_common(prob, qkv, row_stride, t, w, rstd, &np));
+    if (!dqkv || !dw || !workspace) return fail(SA2_ERR_NULL_POINTER, "dqkv, dw or workspace is NULL");
+    if ((reinterpret_cast<uintptr_t>(dqkv) & 15) != 0) return fail(SA2_ERR_ALIGNMENT, "dqkv must be 16-byte aligned");
+    const int64_t need = sa2_qkv_norm_bwd_workspace_bytes(prob);
+    if (workspace_bytes < need)
+        return fail(SA2_ERR_BAD_SHAPE, "workspace of %lld bytes is smaller than the %lld bytes sa2_qkv_norm_bwd_workspace_bytes() asks for",
+                    (long long)workspace_bytes, (long long)need);
+    np.dqkv = static_cast<char *>(dqkv);
+    np.dw_part = static_cast<float *>(workspace);
+    hipStream_t s = static_cast<hipStream_t>(hip_stream);
+    const int groups = norm_groups(prob);
+    const int blocks = groups < kNormMaxBlocks ? groups : kNormMaxBlocks;
+    if (prob->dim_head == 128)
+        hipLaunchKernelGGL(sa2::qkv_norm_bwd_kernel<128>, dim3(blocks), dim3(256), 0, s, np, groups);
+    else
+        hipLaunchKernelGGL(sa2::qkv_norm_bwd_kernel<64>, dim3(blocks), dim3(256), 0, s, np, groups);
+    SA2_TRY(after_launch("qkv norm backward"));
+    const int n = 5 * prob->dim_head;
+    hipLaunchKernelGGL(sa2::qkv_norm_dw_kernel, dim3((n + 255) / 256), dim3(256), 0, s, np.dw_part, dw, blocks, n);
+    return after_launch("qkv norm weight gradients");
 }
 
 }  // extern "C"

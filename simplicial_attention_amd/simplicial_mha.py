@@ -10,6 +10,7 @@ from __future__ import annotations
 from functools import partial
 from typing import Callable
 
+import torch
 from torch import nn
 
 from .naive import naive_two_simplicial_attend
@@ -70,9 +71,26 @@ class HigherOrderAttention(nn.Module):
         t = t.unflatten(-1, (heads, -1))                       # b n h d
         return t.transpose(1, 2) if self.head_first_dim else t
 
+    # fused split + RMSNorm kernel for the layout the sliding-window module uses (GPU, bf16)
+    fused_qkv_norm = True
+
+    def _can_fuse(self, qkv):
+        dh = self.split_dims[0] // self.heads
+        return (self.fused_qkv_norm and self.qk_rmsnorm and self.kv_sets == 2 and not self.head_first_dim
+                and qkv.is_cuda and qkv.dtype is torch.bfloat16 and dh in (64, 128)
+                and self.split_dims[1] == self.split_dims[2]
+                and all(n.eps == self.q_norm.eps for n in (*self.k_norms, *self.v_norms)))
+
     def forward(self, tokens):
         tokens = self.prenorm(tokens)
-        q, k, v = self.to_qkv(tokens).split(self.split_dims, dim=-1)
+        qkv = self.to_qkv(tokens)
+        if qkv.dim() == 3 and self._can_fuse(qkv):
+            from .qkv_norm import fused_qkv_norm
+            norms = (self.q_norm, *self.k_norms, *self.v_norms)
+            q, k1, k2, v1, v2 = fused_qkv_norm(qkv, norms, self.heads, self.key_value_heads, self.split_dims[0] // self.heads)
+            out = self.attend(q, (k1, k2), (v1, v2))
+            return self.postnorm(self.combine_heads(out.flatten(-2)))
+        q, k, v = qkv.split(self.split_dims, dim=-1)
         queries = self._split(q, self.heads)
         keys = self._split(k, self.key_value_heads).chunk(self.kv_sets, dim=-1)
         values = self._split(v, self.key_value_heads).chunk(self.kv_sets, dim=-1)

@@ -61,3 +61,64 @@ def test_module_forward_backward_grouped_heads():
     for name, prm in hip.named_parameters():
         assert prm.grad is not None, name
         assert rel(prm.grad, ref_params[name].grad) <= 3e-2, (name, rel(prm.grad, ref_params[name].grad))
+
+
+@pytest.mark.parametrize('heads,kv_heads,dim_head,n', [(8, 8, 64, 1024), (4, 2, 128, 333)])
+def test_fused_qkv_norm_against_fp32_restatement(heads, kv_heads, dim_head, n):
+    """The fused split + per-head RMSNorm kernel (simplicial_mha.py:116-127 in the reference)
+    against the same arithmetic written with torch in fp32 on the bf16-rounded inputs:
+    outputs within one bf16 rounding, gradients of the projection row and of the five
+    weights through autograd of the restatement."""
+    from simplicial_attention_amd.qkv_norm import FusedQKVNorm
+    g = torch.Generator().manual_seed(7)
+    b, eps = 2, 0.0078125
+    channels = (heads + 4 * kv_heads) * dim_head
+    qkv = torch.randn(b, n, channels, generator=g).bfloat16()
+    ws = [(1 + 0.3 * torch.randn(dim_head, generator=g)).bfloat16() for _ in range(5)]
+    douts = [torch.randn(b, n, h, dim_head, generator=g).bfloat16() for h in (heads, kv_heads, kv_heads, kv_heads, kv_heads)]
+
+    x = qkv.cuda().requires_grad_(True)
+    wd = [w.cuda().requires_grad_(True) for w in ws]
+    outs = FusedQKVNorm.apply(x, *wd, heads, kv_heads, dim_head, eps)
+    torch.autograd.backward(outs, [d.cuda() for d in douts])
+    torch.cuda.synchronize()
+
+    xr = qkv.float().requires_grad_(True)
+    wr = [w.float().requires_grad_(True) for w in ws]
+    qs, ks, vs = xr.split((heads * dim_head, 2 * kv_heads * dim_head, 2 * kv_heads * dim_head), dim=-1)
+    rms = lambda t, w: t * torch.rsqrt(t.pow(2).mean(-1, keepdim=True) + eps) * w
+    k1, k2 = ks.unflatten(-1, (kv_heads, 2 * dim_head)).chunk(2, dim=-1)
+    v1, v2 = vs.unflatten(-1, (kv_heads, 2 * dim_head)).chunk(2, dim=-1)
+    refs = [rms(qs.unflatten(-1, (heads, dim_head)), wr[0]), rms(k1, wr[1]), rms(k2, wr[2]), rms(v1, wr[3]), rms(v2, wr[4])]
+    torch.autograd.backward(refs, [d.float() for d in douts])
+
+    for got, ref in zip(outs, refs):
+        assert got.shape == ref.shape and got.is_contiguous()
+        assert torch.allclose(got.float().cpu(), ref.detach(), atol=1e-6, rtol=2 ** -8)      # one bf16 rounding
+    assert torch.allclose(x.grad.float().cpu(), xr.grad, atol=2e-3, rtol=2 ** -7)
+    for got, ref in zip(wd, wr):
+        rel = float((got.grad.float().cpu() - ref.grad).norm() / ref.grad.norm())
+        assert rel <= 5e-3, rel
+
+
+def test_module_with_and_without_fused_norm_agree():
+    from simplicial_attention_amd import SlidingWindowTwoSimplicialMHA
+    torch.manual_seed(5)
+    m = SlidingWindowTwoSimplicialMHA(256, dim_head=64, heads=4, key_value_heads=2, w1=64, w2=8).bfloat16().cuda()
+    x = torch.randn(2, 150, 256, device='cuda').bfloat16()
+    dout = torch.randn(2, 150, 256, device='cuda').bfloat16()
+
+    def run(fused):
+        m.fused_qkv_norm = fused
+        m.zero_grad()
+        xi = x.clone().requires_grad_(True)
+        out = m(xi)
+        out.backward(dout)
+        return out.detach().float(), xi.grad.float(), {k: v.grad.float() for k, v in m.named_parameters()}
+
+    out_f, dx_f, dp_f = run(True)
+    out_u, dx_u, dp_u = run(False)
+    rel = lambda a, b: float((a - b).norm() / b.norm().clamp_min(1e-30))
+    assert rel(out_f, out_u) <= 1e-2 and rel(dx_f, dx_u) <= 2e-2
+    for k in dp_u:
+        assert rel(dp_f[k], dp_u[k]) <= 2e-2, (k, rel(dp_f[k], dp_u[k]))
