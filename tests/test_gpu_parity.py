@@ -110,3 +110,27 @@ def test_backward_is_deterministic():
         assert torch.equal(first[0], again[0])
         for a, b_ in zip(first[1], again[1]):
             assert torch.equal(a, b_)
+
+
+def test_strided_views_need_no_copy():
+    """q, k1, k2, v1, v2 as interleaved views of one packed (b, n, 5h, d) buffer and a dout view
+    with padded rows: the kernels take the strides as they are (no .contiguous() copy)."""
+    from simplicial_attention_amd import sliding_two_simplicial_attn
+    b, n, h, d, w1, w2 = 2, 300, 2, 128, 128, 16
+    q, k1, k2, v1, v2, dout = U.make_inputs(b, n, h, h, d, seed=31, std=d ** -0.5)
+    packed = torch.stack((q, k1, k2, v1, v2), dim=3).reshape(b, n, h * 5, d).cuda()      # channel (head, tensor)
+    views = [packed.view(b, n, h, 5, d)[:, :, :, x] for x in range(5)]
+    assert not views[0].is_contiguous()
+    dpad = torch.zeros(b, n, h, d + 16, dtype=torch.bfloat16, device='cuda')
+    dpad[..., :d] = dout.cuda()
+    leaves = [v.detach().clone().requires_grad_(True) for v in views]                  # contiguous run
+    out_c = sliding_two_simplicial_attn(leaves[0], (leaves[1], leaves[2]), (leaves[3], leaves[4]), w1=w1, w2=w2)
+    grads_c = torch.autograd.grad(out_c, leaves, dout.cuda())
+    pk = packed.clone().requires_grad_(True)
+    vs = [pk.view(b, n, h, 5, d)[:, :, :, x] for x in range(5)]
+    out_s = sliding_two_simplicial_attn(vs[0], (vs[1], vs[2]), (vs[3], vs[4]), w1=w1, w2=w2)
+    (gpk,) = torch.autograd.grad(out_s, pk, dpad[..., :d])
+    torch.cuda.synchronize()
+    assert torch.equal(out_s, out_c)
+    for x in range(5):
+        assert torch.equal(gpk.view(b, n, h, 5, d)[:, :, :, x], grads_c[x])
