@@ -16,6 +16,8 @@
 // slab hold partial sums that are added once, through LDS, at the end.
 #pragma once
 
+#include <type_traits>
+
 #include "sa2_common.hpp"
 #include "sa2_lds.hpp"
 
@@ -186,7 +188,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
 
     // ---- operand build: threads 0-255 build the even step of a pair, 256-511 the odd one
     const int sub = tid >> 8, t8 = tid & 255;
-    auto build = [&](const Pair &s, int buf) {
+    auto build_by_halves = [&](const Pair &s, int buf) {
         char *stage = lds + buf * L::PAIR + sub * L::STEP;
         const int dlt = 2 * s.m + sub;
         const bool dead = dlt > dmax_of(s.it);        // odd number of offsets: the last pair is half empty
@@ -237,6 +239,63 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
             reinterpret_cast<float *>(stage + L::LSE)[t8] = valid ? reinterpret_cast<const float *>(lds + L::LSES)[t8] : INFINITY;
             if constexpr (DK) reinterpret_cast<float *>(stage + L::DEL)[t8] = valid ? reinterpret_cast<const float *>(lds + L::LSES)[32 + t8] : 0.f;
         }
+    };
+    // D = 128: a tile has 512 pieces, one per thread.  A thread builds ITS piece of both steps
+    // of the pair, so the q (dO) piece is read and unpacked once for two products.
+    auto build_both = [&](const Pair &s, int buf) {
+        const int row = tid / PPR, col = (tid % PPR) * 16;
+        const int dmax = dmax_of(s.it);
+        char *stage = lds + buf * L::PAIR;
+        const int dl0 = 2 * s.m;                                   // never dead
+        const bool dead1 = dl0 + 1 > dmax;
+        const int dl1 = dead1 ? dl0 : dl0 + 1;
+        auto product = [&](int xs, int bs, auto is_a) {             // xs: q or dO rows, bs: k2 or v2 rows
+            constexpr bool IS_A = decltype(is_a)::value;
+            const u32x4 fx = ld_lds16(lds + xs + row * L::RP + col);
+            const u32x4 f0 = ld_lds16(lds + bs + (row - dl0 + L::HALO) * L::RP + col);
+            const u32x4 f1 = ld_lds16(lds + bs + (row - dl1 + L::HALO) * L::RP + col);
+            float xv[8];
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                xv[2 * w] = bf16_lo(fx[w]);
+                xv[2 * w + 1] = bf16_hi(fx[w]);
+            }
+            u32x4 r0, r1;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                r0[w] = pack_bf16(xv[2 * w] * bf16_lo(f0[w]), xv[2 * w + 1] * bf16_hi(f0[w]));
+                r1[w] = pack_bf16(xv[2 * w] * bf16_lo(f1[w]), xv[2 * w + 1] * bf16_hi(f1[w]));
+            }
+            // A: row-major (+ transposed-read copy in the dk1 pass); B: row-major in the dk1 pass, transposed-read in the dv1 pass
+            if (IS_A || DK) {
+                const int o = (IS_A ? L::AS : L::BS) + row * PITCH + col;
+                *reinterpret_cast<u32x4 *>(stage + o) = r0;
+                *reinterpret_cast<u32x4 *>(stage + L::STEP + o) = r1;
+            }
+            if (IS_A == DK) {
+                const int o = L::TR + row * L::TPITCH + col;
+                *reinterpret_cast<u32x4 *>(stage + o) = r0;
+                *reinterpret_cast<u32x4 *>(stage + L::STEP + o) = r1;
+            }
+        };
+        product(L::QS, L::K2S, std::true_type{});
+        if constexpr (DK) __builtin_amdgcn_sched_barrier(0);   // the dk1 pass has no registers for both products at once
+        product(L::DOS, L::V2S, std::false_type{});
+        if (tid < 64) {
+            const int e = tid >> 5, r = tid & 31;
+            const int i = 32 * s.it + r;
+            const int dlt = dl0 + e;
+            const bool valid = dlt <= dmax && i < N && i - dlt >= 0;
+            char *st = stage + e * L::STEP;
+            reinterpret_cast<float *>(st + L::LSE)[r] = valid ? reinterpret_cast<const float *>(lds + L::LSES)[r] : INFINITY;
+            if constexpr (DK) reinterpret_cast<float *>(st + L::DEL)[r] = valid ? reinterpret_cast<const float *>(lds + L::LSES)[32 + r] : 0.f;
+        }
+    };
+    auto build = [&](const Pair &s, int buf) {
+        if constexpr (32 * PPR == 512)
+            build_both(s, buf);
+        else
+            build_by_halves(s, buf);
     };
     auto next_tile = [&](Pair &s) {      // first pair of the next (query head, query tile)
         s.m = 0;
