@@ -242,6 +242,22 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     };
     // D = 128: a tile has 512 pieces, one per thread.  A thread builds ITS piece of both steps
     // of the pair, so the q (dO) piece is read and unpacked once for two products.
+    // dv1 pass: the thread's q and dO pieces stay unpacked in registers for the whole query
+    // tile (the dk1 pass has no registers to spare and unpacks them once per pair)
+    constexpr bool KEEP = !DK && 32 * PPR == 512;
+    float qx[8], ox[8];
+    auto unpack_own = [&]() {
+        const int row = tid / PPR, col = (tid % PPR) * 16;
+        const u32x4 fq = ld_lds16(lds + L::QS + row * L::RP + col);
+        const u32x4 fo = ld_lds16(lds + L::DOS + row * L::RP + col);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            qx[2 * w] = bf16_lo(fq[w]);
+            qx[2 * w + 1] = bf16_hi(fq[w]);
+            ox[2 * w] = bf16_lo(fo[w]);
+            ox[2 * w + 1] = bf16_hi(fo[w]);
+        }
+    };
     auto build_both = [&](const Pair &s, int buf) {
         const int row = tid / PPR, col = (tid % PPR) * 16;
         const int dmax = dmax_of(s.it);
@@ -249,18 +265,11 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
         const int dl0 = 2 * s.m;                                   // never dead
         const bool dead1 = dl0 + 1 > dmax;
         const int dl1 = dead1 ? dl0 : dl0 + 1;
-        auto product = [&](int xs, int bs, auto is_a) {             // xs: q or dO rows, bs: k2 or v2 rows
+        auto product = [&](const float (&xv)[8], int bs, auto is_a) {   // xv: q or dO piece, bs: k2 or v2 rows
             constexpr bool IS_A = decltype(is_a)::value;
-            const u32x4 fx = ld_lds16(lds + xs + row * L::RP + col);
+            u32x4 r0, r1;
             const u32x4 f0 = ld_lds16(lds + bs + (row - dl0 + L::HALO) * L::RP + col);
             const u32x4 f1 = ld_lds16(lds + bs + (row - dl1 + L::HALO) * L::RP + col);
-            float xv[8];
-#pragma unroll
-            for (int w = 0; w < 4; ++w) {
-                xv[2 * w] = bf16_lo(fx[w]);
-                xv[2 * w + 1] = bf16_hi(fx[w]);
-            }
-            u32x4 r0, r1;
 #pragma unroll
             for (int w = 0; w < 4; ++w) {
                 r0[w] = pack_bf16(xv[2 * w] * bf16_lo(f0[w]), xv[2 * w + 1] * bf16_hi(f0[w]));
@@ -278,9 +287,25 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                 *reinterpret_cast<u32x4 *>(stage + L::STEP + o) = r1;
             }
         };
-        product(L::QS, L::K2S, std::true_type{});
-        if constexpr (DK) __builtin_amdgcn_sched_barrier(0);   // the dk1 pass has no registers for both products at once
-        product(L::DOS, L::V2S, std::false_type{});
+        if constexpr (KEEP) {
+            product(qx, L::K2S, std::true_type{});
+            product(ox, L::V2S, std::false_type{});
+        } else {
+            float xv[8];
+            auto unpack = [&](int xs) {
+                const u32x4 fx = ld_lds16(lds + xs + row * L::RP + col);
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    xv[2 * w] = bf16_lo(fx[w]);
+                    xv[2 * w + 1] = bf16_hi(fx[w]);
+                }
+            };
+            unpack(L::QS);
+            product(xv, L::K2S, std::true_type{});
+            __builtin_amdgcn_sched_barrier(0);   // one product at a time: the dk1 pass has no registers for both
+            unpack(L::DOS);
+            product(xv, L::V2S, std::false_type{});
+        }
         if (tid < 64) {
             const int e = tid >> 5, r = tid & 31;
             const int i = 32 * s.it + r;
@@ -313,6 +338,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     write_rows();
     if (rw.g < p.G) issue_rows(rw);
     __syncthreads();
+    if constexpr (KEEP) unpack_own();
     build(nb, 0);
     next_pair(nb);
 
@@ -327,6 +353,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                 next_tile(rw);
                 if (rw.g < p.G) issue_rows(rw);
                 __syncthreads();
+                if constexpr (KEEP) unpack_own();
             }
             TS(1);
             build(nb, (s + 1) & 1);
