@@ -73,7 +73,7 @@ def main():
     ap.add_argument('--workload', default='cfg3_raw_kernel_b4_h8_n8192_d128_w512_w32', choices=sorted(WORKLOADS))
     ap.add_argument('--cpu-slices', type=int, default=4, help='(batch, head) slices of the CPU baseline sample (0 = skip)')
     ap.add_argument('--kernel-iters', type=int, default=5, help='launches per kernel for the per-kernel timing')
-    ap.add_argument('--only', default=None, help='time only this entry through the C ABI (fwd, bwd_delta, bwd_dq_dkv2, bwd_dkv1, bwd_dq_dk2_pass, bwd_dk1_pass, bwd_dv1_pass), `copy`: a 1 GiB device copy that calibrates HBM counters; `module_cfg2`: the module forward of config 2 and the fused qkv-norm kernel; for profiling')
+    ap.add_argument('--only', default=None, help='time only this entry through the C ABI (fwd, bwd_delta, bwd_dq_dkv2, bwd_dkv1, bwd_dq_dk2_pass, bwd_dk1_pass, bwd_dv1_pass), `copy`: a 1 GiB device copy that calibrates HBM counters; `module_cfg2`: the module forward of config 2 and the fused qkv-norm kernel; `train_cfg5`: one training step of the config-5 language model; for profiling')
     args = ap.parse_args()
     if args.gpus != 1:
         print('bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path exists)', file=sys.stderr)
@@ -91,6 +91,51 @@ def main():
 
     B, H, HK, N, D, w1, w2 = WORKLOADS[args.workload]
     dev = torch.device('cuda:0')
+    if args.only == 'train_cfg5':
+        # BASELINE config 5: one training step (forward, loss, backward, Adam) of the byte-level LM: depth 12,
+        # dim 512, 8 heads of 64 (4 key/value heads), every 2nd layer simplicial (w1=512, w2=32), batch 8 x 2048
+        from simplicial_attention_amd.two_simplicial_transformer import TwoSimplicialLM
+        torch.manual_seed(4)
+        lm = TwoSimplicialLM(num_tokens=256, dim=512, depth=12, max_seq_len=2048, dim_head=64, heads=8,
+                             two_simplicial_attn_every=2, transformer_kwargs=dict(key_value_heads=4)).bfloat16().to(dev)
+        opt = torch.optim.Adam(lm.parameters(), lr=1e-4)
+        tokens = torch.randint(0, 256, (8, 2049), device=dev)
+
+        def train_step():
+            opt.zero_grad(set_to_none=True)
+            loss = lm(tokens, return_loss=True)
+            loss.backward()
+            opt.step()
+            return loss
+        for _ in range(max(2, args.warmup)):
+            train_step()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            loss = train_step()
+        torch.cuda.synchronize()
+        step_ms = (time.perf_counter() - t0) / args.steps * 1e3
+        # share of the six simplicial attention cores: the same Function at the layer's shape, timed alone
+        mk5 = lambda h: (torch.randn(8, 2048, h, 64, device=dev) * 0.125).bfloat16().requires_grad_(True)
+        q5, k15, k25, v15, v25 = mk5(8), mk5(4), mk5(4), mk5(4), mk5(4)
+        do5 = torch.randn(8, 2048, 8, 64, device=dev).bfloat16()
+
+        def core():
+            o = sliding_two_simplicial_attn(q5, (k15, k25), (v15, v25), w1=512, w2=32)
+            torch.autograd.grad(o, (q5, k15, k25, v15, v25), do5)
+        for _ in range(3):
+            core()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(10):
+            core()
+        torch.cuda.synchronize()
+        core_ms = (time.perf_counter() - t0) / 10 * 1e3
+        print(json.dumps({'workload': 'cfg5_training_step_depth12_dim512_b8_n2048', 'ms_per_step': round(step_ms, 3),
+                          'tokens_per_s': round(8 * 2048 / step_ms * 1e3, 1), 'loss': round(loss.item(), 4),
+                          'simplicial_core_fwd_bwd_ms_per_layer': round(core_ms, 3),
+                          'simplicial_cores_share_of_step': round(6 * core_ms / step_ms, 3), 'steps': args.steps}))
+        return
     if args.only == 'module_cfg2':
         # BASELINE config 2: the multi-head module, tokens (2, 1024, 512), dim_head 64, 8 heads, forward,
         # with and without the fused split + RMSNorm kernel; and that kernel alone at the config-3 token count
