@@ -186,68 +186,19 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
         }
     };
 
-    // ---- operand build: threads 0-255 build the even step of a pair, 256-511 the odd one
-    const int sub = tid >> 8, t8 = tid & 255;
-    auto build_by_halves = [&](const Pair &s, int buf) {
-        char *stage = lds + buf * L::PAIR + sub * L::STEP;
-        const int dlt = 2 * s.m + sub;
-        const bool dead = dlt > dmax_of(s.it);        // odd number of offsets: the last pair is half empty
-        const int dl = dead ? 0 : dlt;
-        // all LDS reads of a product first, then the multiplies and the writes: the read
-        // latency is paid once per product, not once per piece
-        u32x4 fq[L::LPT], fk[L::LPT];
-        int row[L::LPT], col[L::LPT];
-#pragma unroll
-        for (int x = 0; x < L::LPT; ++x) {
-            const int pc = x * 256 + t8;
-            row[x] = pc / PPR;
-            col[x] = (pc % PPR) * 16;
-            fq[x] = ld_lds16(lds + L::QS + row[x] * L::RP + col[x]);
-            fk[x] = ld_lds16(lds + L::K2S + (row[x] - dl + L::HALO) * L::RP + col[x]);
-        }
-        u32x4 fo[L::LPT], fv[L::LPT];
-        if constexpr (DK) __builtin_amdgcn_sched_barrier(0);   // the dk1 pass has no registers for both products at once
-#pragma unroll
-        for (int x = 0; x < L::LPT; ++x) {
-            if constexpr (!DK) {
-                fo[x] = ld_lds16(lds + L::DOS + row[x] * L::RP + col[x]);
-                fv[x] = ld_lds16(lds + L::V2S + (row[x] - dl + L::HALO) * L::RP + col[x]);
-            }
-        }
-#pragma unroll
-        for (int x = 0; x < L::LPT; ++x) {
-            const u32x4 a = mul_bf16x8(fq[x], fk[x]);
-            *reinterpret_cast<u32x4 *>(stage + L::AS + row[x] * PITCH + col[x]) = a;
-            if constexpr (DK) *reinterpret_cast<u32x4 *>(stage + L::TR + row[x] * L::TPITCH + col[x]) = a;
-        }
-        if constexpr (DK) {
-            __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-            for (int x = 0; x < L::LPT; ++x) {
-                fo[x] = ld_lds16(lds + L::DOS + row[x] * L::RP + col[x]);
-                fv[x] = ld_lds16(lds + L::V2S + (row[x] - dl + L::HALO) * L::RP + col[x]);
-            }
-        }
-#pragma unroll
-        for (int x = 0; x < L::LPT; ++x) {
-            const u32x4 bb = mul_bf16x8(fo[x], fv[x]);
-            *reinterpret_cast<u32x4 *>(stage + (DK ? L::BS + row[x] * PITCH : L::TR + row[x] * L::TPITCH) + col[x]) = bb;
-        }
-        if (t8 < 32) {
-            const int i = 32 * s.it + t8;
-            const bool valid = !dead && i < N && i - dlt >= 0;
-            reinterpret_cast<float *>(stage + L::LSE)[t8] = valid ? reinterpret_cast<const float *>(lds + L::LSES)[t8] : INFINITY;
-            if constexpr (DK) reinterpret_cast<float *>(stage + L::DEL)[t8] = valid ? reinterpret_cast<const float *>(lds + L::LSES)[32 + t8] : 0.f;
-        }
-    };
-    // D = 128: a tile has 512 pieces, one per thread.  A thread builds ITS piece of both steps
+    // ---- operand build.  A tile has 32 * D/8 pieces of 16 bytes: 512 at D = 128, one per
+    // thread, and a thread builds its piece of A and of B; 256 at D = 64, where threads 0-255
+    // build A and threads 256-511 build B.  Either way a thread builds ITS piece for both steps
     // of the pair, so the q (dO) piece is read and unpacked once for two products.
     // dv1 pass: the thread's q and dO pieces stay unpacked in registers for the whole query
     // tile (the dk1 pass has no registers to spare and unpacks them once per pair)
-    constexpr bool KEEP = !DK && 32 * PPR == 512;
+    constexpr int PIECES = 32 * PPR;
+    constexpr bool BOTH = PIECES == 512;
+    constexpr bool KEEP = !DK && BOTH;
+    const int b_row = (tid % PIECES) / PPR, b_col = (tid % PPR) * 16;
     float qx[8], ox[8];
     auto unpack_own = [&]() {
-        const int row = tid / PPR, col = (tid % PPR) * 16;
+        const int row = b_row, col = b_col;
         const u32x4 fq = ld_lds16(lds + L::QS + row * L::RP + col);
         const u32x4 fo = ld_lds16(lds + L::DOS + row * L::RP + col);
 #pragma unroll
@@ -258,8 +209,8 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
             ox[2 * w + 1] = bf16_hi(fo[w]);
         }
     };
-    auto build_both = [&](const Pair &s, int buf) {
-        const int row = tid / PPR, col = (tid % PPR) * 16;
+    auto build = [&](const Pair &s, int buf) {
+        const int row = b_row, col = b_col;
         const int dmax = dmax_of(s.it);
         char *stage = lds + buf * L::PAIR;
         const int dl0 = 2 * s.m;                                   // never dead
@@ -300,11 +251,15 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                     xv[2 * w + 1] = bf16_hi(fx[w]);
                 }
             };
-            unpack(L::QS);
-            product(xv, L::K2S, std::true_type{});
-            __builtin_amdgcn_sched_barrier(0);   // one product at a time: the dk1 pass has no registers for both
-            unpack(L::DOS);
-            product(xv, L::V2S, std::false_type{});
+            if (BOTH || tid < PIECES) {
+                unpack(L::QS);
+                product(xv, L::K2S, std::true_type{});
+            }
+            if constexpr (BOTH) __builtin_amdgcn_sched_barrier(0);   // one product at a time: the dk1 pass has no registers for both
+            if (BOTH || tid >= PIECES) {
+                unpack(L::DOS);
+                product(xv, L::V2S, std::false_type{});
+            }
         }
         if (tid < 64) {
             const int e = tid >> 5, r = tid & 31;
@@ -315,12 +270,6 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
             reinterpret_cast<float *>(st + L::LSE)[r] = valid ? reinterpret_cast<const float *>(lds + L::LSES)[r] : INFINITY;
             if constexpr (DK) reinterpret_cast<float *>(st + L::DEL)[r] = valid ? reinterpret_cast<const float *>(lds + L::LSES)[32 + r] : 0.f;
         }
-    };
-    auto build = [&](const Pair &s, int buf) {
-        if constexpr (32 * PPR == 512)
-            build_both(s, buf);
-        else
-            build_by_halves(s, buf);
     };
     auto next_tile = [&](Pair &s) {      // first pair of the next (query head, query tile)
         s.m = 0;
