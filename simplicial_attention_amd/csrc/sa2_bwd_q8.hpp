@@ -223,9 +223,12 @@ __global__ __launch_bounds__(512) void bwd_q8_kernel(KParams p, float *ws) {
 
         const char *stage = lds;
         auto sync_stage = [&]() {
+            // stage u goes into its buffer (last read in step u-2) before the barrier that publishes it
+            if (u >= 1 && u_load - 1 >= u) {
+                write_stage(u & 1);
+                if (u_load < U) issue_loads();
+            }
             __syncthreads();
-            if (u_load - 1 > u) write_stage((u + 1) & 1);
-            if (u_load < U) issue_loads();
             stage = lds + (u & 1) * C::STAGE;
             ++u;
         };

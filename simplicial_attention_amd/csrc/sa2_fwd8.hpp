@@ -171,8 +171,8 @@ __global__ __launch_bounds__(512) void fwd8_kernel(KParams p) {
     float seen = -INFINITY;    // running maximum of x relative to M; -inf: no valid entry yet
     float l = 0.f;
 
-    // ring protocol: the stage of step u+1 is written right after the barrier of step u (its
-    // buffer was last read in step u-1), from registers loaded during step u-1
+    // ring protocol: stage u is written right before the barrier of step u (its buffer was last
+    // read in step u-2), from registers loaded right before the barrier of step u-1
     issue_loads();
     write_stage(0);
     if (U > 1) issue_loads();
@@ -279,10 +279,14 @@ __global__ __launch_bounds__(512) void fwd8_kernel(KParams p) {
         // barrier + refill of the ring behind the stage that becomes current
         auto sync_stage = [&]() {
             TS(3);
+            // stage u goes into its buffer (last read in step u-2) BEFORE the barrier that
+            // publishes it: the writes fall into the time a wave would otherwise wait for the others
+            if (u >= 1 && u_load - 1 >= u) {
+                write_stage(u & 1);
+                if (u_load < U) issue_loads();
+            }
             __syncthreads();
             TS(0);
-            if (u_load - 1 > u) write_stage((u + 1) & 1);
-            if (u_load < U) issue_loads();
             stage = lds + (u & 1) * C::STAGE;
             ++u;
             TS(1);
