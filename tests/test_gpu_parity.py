@@ -19,6 +19,8 @@ CASES = [
     (1, 300, 2, 1, 64, 100, 33),      # windows not multiples of 32, w2 > 32
     (1, 640, 2, 2, 128, 512, 32),     # default windows, D = 128
     (1, 1000, 2, 2, 64, 512, 32),     # ragged N with the default windows
+    (1, 150, 2, 2, 128, 40, 5),       # odd number of offsets: the last offset pair of a step is half empty
+    (1, 260, 2, 1, 128, 70, 64),      # widest second window, D = 128 (fused four-wave backward kernels)
 ]
 
 
