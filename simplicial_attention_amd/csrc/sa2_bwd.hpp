@@ -50,28 +50,6 @@ __global__ __launch_bounds__(256) void delta_kernel(KParams p) {
     if (ok && piece == 0) p.delta[row] = s;
 }
 
-// small GEMM helpers ---------------------------------------------------------------------
-
-// acc(32x32, rows = staged rows, column = lane column) = sum_kk lds_rows[kk] * regfrag[kk]
-template <int KS>
-__device__ __forceinline__ f32x16 gemm_rows(const char *lds_row_base, const u32x4 (&frag)[KS]) {
-    f32x16 s = zero16();
-#pragma unroll
-    for (int kk = 0; kk < KS; ++kk) s = mfma32(ld_lds16(lds_row_base + 32 * kk), frag[kk], s);
-    return s;
-}
-
-// acc[dt](rows = d, column = lane column) += transposed-chunk rows * packed C-layout fragment
-template <int DT>
-__device__ __forceinline__ void gemm_trans(f32x16 (&acc)[DT], const char *tbase, int pitch, const u32x4 (&pb)[2]) {
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt) {
-        const char *b = tbase + 32 * dt * pitch;
-        acc[dt] = mfma32(ld_lds16(b), pb[0], acc[dt]);
-        acc[dt] = mfma32(ld_lds16(b + 32), pb[1], acc[dt]);
-    }
-}
-
 // ------------------------------------------------------------------------------------
 // dK1/dV1: workgroup = 128 rows j of one (batch, kv head); wave w owns rows
 // [32w, 32w+32), lane column = j, and keeps its K1/V1 fragments in registers as B

@@ -399,7 +399,7 @@ __global__ __launch_bounds__(256) void dv2_from_saved_kernel(KParams p) {
         const int64_t bh_row = ((int64_t)b * p.H + h);
         const char *dog = p.dout.ptr + b * p.dout.sb + h * p.dout.sh + col;
         const float *lse = p.lse + bh_row * N;
-#pragma unroll 4
+#pragma unroll 8
         for (int dlt = 0; dlt < nd; ++dlt) {
             const int i = k + dlt;
             const int64_t srow = (bh_row * p.w2 + dlt) * N + i;

@@ -70,25 +70,10 @@ __device__ __forceinline__ u32x4 mul_bf16x8(u32x4 a, u32x4 b) {
     return r;
 }
 
-// a * b * s, one rounding to bf16
-__device__ __forceinline__ u32x4 mul_bf16x8_scaled(u32x4 a, u32x4 b, float s) {
-    u32x4 r;
-#pragma unroll
-    for (int w = 0; w < 4; ++w) r[w] = pack_bf16(bf16_lo(a[w]) * bf16_lo(b[w]) * s, bf16_hi(a[w]) * bf16_hi(b[w]) * s);
-    return r;
-}
-
 // c + lo(x) + hi(x) for a packed pair of bf16 (v_dot2c_f32_bf16 against (1, 1))
 __device__ __forceinline__ float add_bf16x2(uint32_t x, float c) {
     typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
     return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, x), __builtin_bit_cast(bf16x2_t, 0x3f803f80u), c, false);
-}
-
-__device__ __forceinline__ f32x16 splat16(float v) {
-    f32x16 r;
-#pragma unroll
-    for (int i = 0; i < 16; ++i) r[i] = v;
-    return r;
 }
 
 // wave index as a scalar: branches on it are uniform and index arithmetic stays on the scalar unit
@@ -111,72 +96,16 @@ __device__ __forceinline__ f32x16 zero16() {
     return z;
 }
 
-// value held by the lane with the same column in the other half of the wave
-__device__ __forceinline__ float other_half(float x) { return __shfl_xor(x, 32, 64); }
+
 
 __device__ __forceinline__ bool wave_any(bool pred) { return __builtin_amdgcn_ballot_w64(pred) != 0ull; }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
-// Storage position of row j (0..15 within an aligned group of 16) inside a
-// "k-slot ordered" transposed tile: rows 8a+4h+c (a,h in {0,1}, c in 0..3) sit at
-// 8h+4a+c, so that the 8 rows a C-layout lane of half h owns are contiguous.
-__device__ __forceinline__ int kslot_pos(int j) {
-    return (j & ~15) | ((j & 4) << 1) | ((j & 8) >> 1) | (j & 3);
-}
-
 // d index (within a 32-wide d tile) handled by MFMA row c of a "transposed output"
 // GEMM (output rows = d), chosen so that the 16 accumulator registers of a lane
 // cover 16 consecutive d:  register r of half hf  <->  d = 16*hf + r.
 __device__ __forceinline__ int dmap_row(int c) { return 16 * ((c >> 2) & 1) + 4 * (c >> 3) + (c & 3); }
-
-// ---- LDS staging of a 128-row chunk of a (seq, dim) matrix, 256 threads ----------
-constexpr int kChunkTiles = 4;                       // 32-row tiles per chunk (= waves)
-constexpr int kChunkRows = kChunkTiles * 32;
-constexpr int kChunkPitchT = (kChunkRows + 8) * 2;   // pitch of a transposed chunk row
-__host__ __device__ constexpr int row_pitch(int d) { return (d + 8) * 2; }  // padded row-major pitch
-
-// Row-major copy: dst[row][d], rows row0 .. row0+127 of src; rows >= N are zero.
-template <int D>
-__device__ __forceinline__ void stage_rows(char *dst, const char *src, int64_t sn, int row0, int N) {
-    constexpr int PPR = D / 8;  // 16-byte pieces per row
-    const int tid = threadIdx.x;
-#pragma unroll
-    for (int it = 0; it < kChunkRows * PPR / 256; ++it) {
-        int idx = it * 256 + tid;
-        int row = idx / PPR, piece = idx % PPR;
-        int j = row0 + row;
-        u32x4 v = {0u, 0u, 0u, 0u};
-        if (j < N) v = ld_global16(src + (int64_t)j * sn + piece * 16);
-        *reinterpret_cast<u32x4 *>(dst + row * row_pitch(D) + piece * 16) = v;
-    }
-}
-
-// Transposed copy: dst[d][kslot_pos(row)], so that a lane of half hf reads the 8 rows
-// it needs for one k-step (16 rows) of a GEMM contracting over rows as one 16-byte word.
-template <int D>
-__device__ __forceinline__ void stage_rows_transposed(char *dst, const char *src, int64_t sn, int row0, int N) {
-    const int tid = threadIdx.x;
-    const int wave = tid >> 6, lane = tid & 63;
-    constexpr int LPR = D / 2;     // lanes covering one row with 4-byte loads
-    constexpr int GPW = 64 / LPR;  // 4-row groups per wave instruction
-    const int dpair = lane % LPR;
-#pragma unroll
-    for (int it = 0; it < 8 / GPW; ++it) {
-        int rl0 = 32 * wave + 4 * (it * GPW + lane / LPR);
-        uint32_t w[4];
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            int j = row0 + rl0 + r;
-            w[r] = (j < N) ? *reinterpret_cast<const uint32_t *>(src + (int64_t)j * sn + dpair * 4) : 0u;
-        }
-        u32x2 lo = {(w[0] & 0xffffu) | (w[1] << 16), (w[2] & 0xffffu) | (w[3] << 16)};
-        u32x2 hi = {(w[0] >> 16) | (w[1] & 0xffff0000u), (w[2] >> 16) | (w[3] & 0xffff0000u)};
-        int pos = kslot_pos(rl0);
-        *reinterpret_cast<u32x2 *>(dst + (2 * dpair) * kChunkPitchT + pos * 2) = lo;
-        *reinterpret_cast<u32x2 *>(dst + (2 * dpair + 1) * kChunkPitchT + pos * 2) = hi;
-    }
-}
 
 // acc[dt][r] += x[32*dt + 16*hf + r] * g[dt][r]; xrow points at element 16*hf of the row
 template <int DT>
