@@ -51,7 +51,7 @@ class HigherOrderAttention(nn.Module):
         if qk_rmsnorm:
             self.q_norm = nn.RMSNorm(dim_head)
             self.k_norms = nn.ModuleList(nn.RMSNorm(dim_head) for _ in range(self.kv_sets))
-            self.v_norms = nn.ModuleList(nn.RMSNorm(dim_head) for _ in range(self.kv_sets))
+            self.v_norms = nn.ModuleList(nn.RMSNorm(dim_head_values) for _ in range(self.kv_sets))
 
         self.split_dims = (heads * dim_head,
                            self.kv_sets * key_value_heads * dim_head,

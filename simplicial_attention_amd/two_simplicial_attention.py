@@ -13,6 +13,7 @@ import os
 from functools import partial
 
 import torch
+import torch.nn.functional as F
 from torch import Tensor
 from torch.autograd import Function
 
@@ -38,16 +39,19 @@ def save_partials_max_bytes() -> int:
 
 
 class SlidingTwoSimplicialAttention(Function):
-    """``apply(q, k1, k2, v1, v2, w1, w2, causal) -> out``; every tensor ``(b, n, h, d)``.
+    """``apply(q, k1, k2, v1, v2, w1, w2, causal[, scale]) -> out``; every tensor ``(b, n, h, d)``.
 
     ``k1, k2, v1, v2`` may carry fewer heads than ``q`` (grouped queries, query head
     ``h`` reads key/value head ``h // groups``); the reference's Function receives
     them already repeated, which is the special case of one group per head.
     Gradients come back in the order ``dq, dk1, dk2, dv1, dv2`` in the input dtype.
+    ``scale`` (not an argument of the reference's Function, which always uses
+    ``dim_head ** -0.5``) overrides the softmax scale; the functional wrapper passes it
+    when it has zero-padded the head dimension.
     """
 
     @staticmethod
-    def forward(ctx, q, k1, k2, v1, v2, w1, w2, causal):
+    def forward(ctx, q, k1, k2, v1, v2, w1, w2, causal, scale=None):
         tensors = (q, k1, k2, v1, v2)
         assert all(t.is_cuda for t in tensors), 'sliding-window 2-simplicial attention runs on the GPU only'
         if not causal:
@@ -71,7 +75,7 @@ class SlidingTwoSimplicialAttention(Function):
             raise NotImplementedError(f'dim_head={dim}, w1={w1}, w2={w2} is not covered by the kernels (dim_head 64 or 128, w2 <= 64)')
 
         q, k1, k2, v1, v2 = (_unit_inner_stride(t) for t in tensors)
-        scale = dim ** -0.5
+        scale = dim ** -0.5 if scale is None else float(scale)
         out = torch.empty((batch, seq_len, heads, dim), dtype=q.dtype, device=q.device)
         lse = torch.empty((batch, heads, seq_len), dtype=torch.float32, device=q.device)
         # bf16 residual of the fp32 accumulator, kept only when a backward may follow
@@ -115,7 +119,7 @@ class SlidingTwoSimplicialAttention(Function):
                                       delta.data_ptr(),
                                       arg(dq), arg(dk1), arg(dk2), arg(dv1), arg(dv2),
                                       workspace.data_ptr(), ws_bytes, _stream_handle(q.device)))
-        return dq, dk1, dk2, dv1, dv2, None, None, None
+        return dq, dk1, dk2, dv1, dv2, None, None, None, None
 
 
 _sliding_two_simplicial_attn = SlidingTwoSimplicialAttention.apply
@@ -136,13 +140,38 @@ def sliding_two_simplicial_attn(
     ragged sequence end is masked there, so nothing is repeated or padded here;
     ``pad_to_multiple_of`` is accepted for compatibility and has no effect on the
     result (zero rows appended after a causal sequence cannot influence it).
+
+    Beyond the reference (whose kernels are written for bf16 and a head dimension of
+    64): float16 and float32 tensors are computed in bfloat16 and the result returned
+    in the input dtype; any head dimension up to 128, and a value head dimension
+    different from the query/key one, are zero-padded to the kernels' 64 or 128
+    (padded query/key channels add nothing to the logits, padded value channels give
+    zero outputs that are sliced off; the softmax scale stays that of the true
+    query/key dimension).
     """
     if len(keys) != 2 or len(values) != 2:
         raise AssertionError('two key sets and two value sets are required')
     q_heads, k_heads = q.shape[-2], keys[0].shape[-2]
     assert q_heads % k_heads == 0, 'query heads must be a multiple of key/value heads'
     (k1, k2), (v1, v2) = keys, values
-    return _sliding_two_simplicial_attn(q, k1, k2, v1, v2, w1, w2, causal)
+    dtype, dim_qk, dim_v = q.dtype, q.shape[-1], v1.shape[-1]
+    if dtype not in (torch.bfloat16, torch.float16, torch.float32):
+        raise TypeError(f'unsupported dtype {dtype}')
+    if k1.shape[-1] != dim_qk or k2.shape[-1] != dim_qk or v2.shape[-1] != dim_v:
+        raise ValueError('q, k1, k2 must share one head dimension and v1, v2 another')
+    dim = max(dim_qk, dim_v)
+    if dim > 128:
+        raise NotImplementedError(f'head dimension {dim} is not covered by the kernels (at most 128)')
+    if dtype is torch.bfloat16 and dim_qk == dim_v and dim in (64, 128):
+        return _sliding_two_simplicial_attn(q, k1, k2, v1, v2, w1, w2, causal)
+    dim_kernel = 64 if dim <= 64 else 128
+
+    def prepare(t):
+        t = t.to(torch.bfloat16)
+        return F.pad(t, (0, dim_kernel - t.shape[-1])) if t.shape[-1] != dim_kernel else t
+
+    out = _sliding_two_simplicial_attn(*(prepare(t) for t in (q, k1, k2, v1, v2)), w1, w2, causal, dim_qk ** -0.5)
+    return out[..., :dim_v].to(dtype)
 
 
 class SlidingWindowTwoSimplicialMHA(HigherOrderAttention):

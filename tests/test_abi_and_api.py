@@ -101,6 +101,29 @@ def test_function_rejects_what_the_kernels_do_not_cover():
         S.sliding_two_simplicial_attn(torch.randn(1, 16, 3, 64), (q, q), (q, q))
 
 
+def test_wrapper_checks_head_dimensions_and_dtypes():
+    q = torch.randn(1, 16, 2, 64)
+    wide = torch.randn(1, 16, 2, 160)
+    with pytest.raises(NotImplementedError):     # beyond the kernels' largest head dimension
+        S.sliding_two_simplicial_attn(wide, (wide, wide), (wide, wide))
+    with pytest.raises(ValueError):              # k2 with a head dimension of its own
+        S.sliding_two_simplicial_attn(q, (q, q[..., :32]), (q, q))
+    with pytest.raises(ValueError):
+        S.sliding_two_simplicial_attn(q, (q, q), (q, q[..., :32]))
+    with pytest.raises(TypeError):
+        S.sliding_two_simplicial_attn(q.double(), (q.double(),) * 2, (q.double(),) * 2)
+
+
+def test_module_with_a_value_head_dimension_of_its_own():
+    """dim_head_values (simplicial_mha.py:34,56 of the reference) sizes the value part of the
+    projection, the value norms and the output projection."""
+    m = S.HigherOrderAttention(dim=64, dim_head=16, dim_head_values=8, heads=2, key_value_heads=1, causal=True)
+    assert m.to_qkv.weight.shape == (2 * 16 + 2 * 16 + 2 * 8, 64)
+    assert m.combine_heads.weight.shape == (64, 2 * 8)
+    assert m.v_norms[0].weight.shape == (8,) and m.k_norms[0].weight.shape == (16,)
+    assert m(torch.randn(2, 10, 64)).shape == (2, 10, 64)
+
+
 def test_module_mirrors_reference_constructor_and_parameters():
     m = S.SlidingWindowTwoSimplicialMHA(dim=512, dim_head=64, heads=8)
     sd = m.state_dict()

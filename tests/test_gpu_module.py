@@ -9,14 +9,15 @@ from oracle import reference_attend as R
 pytestmark = pytest.mark.gpu
 
 
-def _pair(dim, heads, kv_heads, dim_head, w1, w2, seed):
+def _pair(dim, heads, kv_heads, dim_head, w1, w2, seed, dim_head_values=None):
     from simplicial_attention_amd import SlidingWindowTwoSimplicialMHA
     from simplicial_attention_amd.simplicial_mha import HigherOrderAttention
     torch.manual_seed(seed)
-    hip = SlidingWindowTwoSimplicialMHA(dim, dim_head=dim_head, heads=heads, key_value_heads=kv_heads, w1=w1, w2=w2)
+    hip = SlidingWindowTwoSimplicialMHA(dim, dim_head=dim_head, heads=heads, key_value_heads=kv_heads, w1=w1, w2=w2,
+                                        dim_head_values=dim_head_values)
     attend = lambda q, k, v: R.sliding_two_simplicial_attn(q, k, v, w1=w1, w2=w2)
     ref = HigherOrderAttention(dim, dim_head=dim_head, heads=heads, key_value_heads=kv_heads, attend=attend,
-                               head_first_dim=False)
+                               head_first_dim=False, dim_head_values=dim_head_values)
     ref.load_state_dict(hip.state_dict())
     # the oracle module computes in fp32 on the bf16-rounded weights
     hip = hip.bfloat16()
@@ -61,6 +62,25 @@ def test_module_forward_backward_grouped_heads():
     for name, prm in hip.named_parameters():
         assert prm.grad is not None, name
         assert rel(prm.grad, ref_params[name].grad) <= 3e-2, (name, rel(prm.grad, ref_params[name].grad))
+
+
+def test_module_with_narrow_value_heads_and_small_query_heads():
+    """dim_head 32 with dim_head_values 16 (simplicial_mha.py:34,56 in the reference): the
+    module takes the unfused norm path and the wrapper pads both to the kernels' 64."""
+    hip, ref = _pair(128, 4, 2, 32, 64, 8, seed=5, dim_head_values=16)
+    g = torch.Generator().manual_seed(6)
+    tokens = torch.randn(2, 150, 128, generator=g).bfloat16()
+    dout = torch.randn(2, 150, 128, generator=g).bfloat16()
+    x_hip = tokens.cuda().requires_grad_(True)
+    out = hip(x_hip)
+    out.backward(dout.cuda())
+    x_ref = tokens.float().requires_grad_(True)
+    want = ref(x_ref)
+    want.backward(dout.float())
+    torch.cuda.synchronize()
+    rel = lambda a, b: float((a.float().cpu() - b).norm() / b.norm().clamp_min(1e-30))
+    assert rel(out.detach(), want.detach()) <= 2e-2
+    assert rel(x_hip.grad, x_ref.grad) <= 3e-2
 
 
 @pytest.mark.parametrize('heads,kv_heads,dim_head,n', [(8, 8, 64, 1024), (4, 2, 128, 333)])

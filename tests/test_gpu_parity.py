@@ -104,6 +104,33 @@ def test_backward_that_recomputes_instead_of_using_saved_partials(shape, monkeyp
     U.check_all(out, grads, ref_out, ref_grads)
 
 
+@pytest.mark.parametrize('dtype,dqk,dv,n,w1,w2', [
+    (torch.float32, 32, 32, 128, 128, 64),     # head size and dtype of the reference's CPU-runnable case
+    (torch.bfloat16, 64, 32, 200, 64, 16),     # value heads narrower than query/key heads
+    (torch.float16, 48, 128, 150, 40, 8),      # neither 64 nor 128; value heads wider
+    (torch.bfloat16, 96, 96, 100, 512, 32),
+])
+def test_other_head_dimensions_and_dtypes(dtype, dqk, dv, n, w1, w2):
+    """Head dimensions other than 64/128, a value head dimension of its own, and float16 /
+    float32 tensors: the functional wrapper pads and casts around the bf16 kernels; output
+    and gradients come back in the caller's dtype and shapes.  The oracle works on the
+    bf16-rounded values with the scale of the true query/key dimension."""
+    from simplicial_attention_amd import sliding_two_simplicial_attn
+    b, hq, hk = 1, 4, 2
+    g = torch.Generator(device='cpu').manual_seed(dqk + dv)
+    rnd = lambda h, d: torch.randn(b, n, h, d, generator=g).bfloat16()
+    q, k1, k2 = rnd(hq, dqk), rnd(hk, dqk), rnd(hk, dqk)
+    v1, v2, dout = rnd(hk, dv), rnd(hk, dv), rnd(hq, dv)
+    ref_out, _, ref_grads = U.oracle_fwd_bwd(q, k1, k2, v1, v2, dout, w1, w2)
+    ts = [t.to(dtype).cuda().requires_grad_(True) for t in (q, k1, k2, v1, v2)]
+    out = sliding_two_simplicial_attn(ts[0], (ts[1], ts[2]), (ts[3], ts[4]), w1=w1, w2=w2)
+    assert out.dtype is dtype and out.shape == (b, n, hq, dv)
+    grads = torch.autograd.grad(out, ts, dout.to(dtype).cuda())
+    for got, leaf in zip(grads, ts):
+        assert got.dtype is dtype and got.shape == leaf.shape
+    U.check_all(out, grads, ref_out, ref_grads, unit_variance=True)
+
+
 def test_backward_is_deterministic():
     ins = U.make_inputs(1, 384, 2, 1, 128, seed=11)
     first = U.hip_fwd_bwd(*ins, 128, 32)
