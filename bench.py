@@ -258,8 +258,9 @@ def main():
                     del os.environ['SA2_BWD_PASS']
             return run
         launches['bwd_dq_dk2_pass'] = (3, one_pass('first', launches['bwd_dq_dkv2'][1]))
-        launches['bwd_dk1_pass'] = (3, one_pass('first', launches['bwd_dkv1'][1]))
-        launches['bwd_dv1_pass'] = (2, one_pass('second', launches['bwd_dkv1'][1]))
+        if D == 128:         # at dim_head 64 one kernel produces dK1 and dV1 (bwd_dkv1 is a single launch)
+            launches['bwd_dk1_pass'] = (3, one_pass('first', launches['bwd_dkv1'][1]))
+            launches['bwd_dv1_pass'] = (2, one_pass('second', launches['bwd_dkv1'][1]))
     kernels = {}
     if args.only is not None:
         # the later kernels read what the earlier ones wrote: run the chain once, untimed
@@ -287,11 +288,14 @@ def main():
         return
     hbm_bytes = {'fwd': 7 * B * N * H * D * 2 + 4 * B * H * N, 'bwd_delta': 3 * B * N * H * D * 2 + 4 * B * H * N}
     # entries that are exactly one kernel launch (the two-pass entry points are timed per pass)
-    single = [k for k in kernels if kernels[k]['contractions'] and (w2 > 32 or k not in ('bwd_dq_dkv2', 'bwd_dkv1'))]
+    multi = () if w2 > 32 else ('bwd_dq_dkv2', 'bwd_dkv1') if D == 128 else ('bwd_dq_dkv2',)
+    single = [k for k in kernels if kernels[k]['contractions'] and k not in multi]
     dom = max(single, key=lambda k: kernels[k]['ms'])
     achieved = kernels[dom]['tflops']
     symbols = {'fwd': 'sa2::fwd8_kernel<%d>' % D, 'bwd_dq_dk2_pass': 'sa2::bwd_q8_kernel<%d, true>' % D,
-               'bwd_dk1_pass': 'sa2::bwd_kv8_kernel<%d, true>' % D, 'bwd_dv1_pass': 'sa2::bwd_kv8_kernel<%d, false>' % D}
+               'bwd_dk1_pass': 'sa2::bwd_kv8_kernel<%d, 1>' % D, 'bwd_dv1_pass': 'sa2::bwd_kv8_kernel<%d, 0>' % D}
+    if D == 64 and w2 <= 32:
+        symbols['bwd_dkv1'] = 'sa2::bwd_kv8_kernel<64, 2>'
     # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `--only <entry>` on this
     # workload, scaled by what the same counters read for a 1 GiB device copy (profiles/pmc_cfg3_mfma_kernels.txt)
     measured_traffic = {

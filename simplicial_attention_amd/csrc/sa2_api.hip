@@ -308,17 +308,23 @@ int sa2_bwd_dkv1(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor 
 #endif
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
     int grid = prob->batch * prob->kv_heads * ((prob->seq_len + 127) / 128);
-    // offsets up to 32: two eight-wave passes (dk1, then dv1); wider second windows (or
-    // SA2_BWD_KV1_IMPL=fused) take the fused four-wave kernel
+    // offsets up to 32: eight-wave kernels, two passes (dk1, then dv1) at dim_head 128 and one
+    // kernel for both at dim_head 64; wider second windows (or SA2_BWD_KV1_IMPL=fused) take the
+    // fused four-wave kernel
     const char *impl = std::getenv("SA2_BWD_KV1_IMPL");
     const bool fused = prob->w2 > 32 || (impl && std::strcmp(impl, "fused") == 0);
     const int pass = bwd_pass_filter();
     if (!fused && prob->dim_head == 128) {
-        if (pass != 2) hipLaunchKernelGGL((sa2::bwd_kv8_kernel<128, true>), dim3(grid), dim3(512), 0, s, k);
-        if (pass != 1) hipLaunchKernelGGL((sa2::bwd_kv8_kernel<128, false>), dim3(grid), dim3(512), 0, s, k);
+        if (pass != 2) hipLaunchKernelGGL((sa2::bwd_kv8_kernel<128, sa2::kKvDk>), dim3(grid), dim3(512), 0, s, k);
+        if (pass != 1) hipLaunchKernelGGL((sa2::bwd_kv8_kernel<128, sa2::kKvDv>), dim3(grid), dim3(512), 0, s, k);
     } else if (!fused) {
-        if (pass != 2) hipLaunchKernelGGL((sa2::bwd_kv8_kernel<64, true>), dim3(grid), dim3(512), 0, s, k);
-        if (pass != 1) hipLaunchKernelGGL((sa2::bwd_kv8_kernel<64, false>), dim3(grid), dim3(512), 0, s, k);
+        const char *split = std::getenv("SA2_BWD_KV1_SPLIT");       // profiling knob: the two passes at dim_head 64 too
+        if (split && split[0] == '1') {
+            if (pass != 2) hipLaunchKernelGGL((sa2::bwd_kv8_kernel<64, sa2::kKvDk>), dim3(grid), dim3(512), 0, s, k);
+            if (pass != 1) hipLaunchKernelGGL((sa2::bwd_kv8_kernel<64, sa2::kKvDv>), dim3(grid), dim3(512), 0, s, k);
+        } else {
+            hipLaunchKernelGGL((sa2::bwd_kv8_kernel<64, sa2::kKvBoth>), dim3(grid), dim3(512), 0, s, k);
+        }
     } else if (prob->dim_head == 128)
         hipLaunchKernelGGL(sa2::bwd_dkv1_kernel<128>, dim3(grid), dim3(256), 0, s, k);
     else

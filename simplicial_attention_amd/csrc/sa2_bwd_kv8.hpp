@@ -6,11 +6,12 @@
 // offset and the waves of group 1 the odd one.  The q/do rows of a query tile and the 63
 // k2/v2 rows its offsets (at most 32) can reach are staged in LDS once per tile; from
 // them the 512 threads build A = q*k2 and B = do*v2 of both steps once per barrier.  A fused kernel (dK1 and dV1
-// accumulators, K1 and V1 fragments) needs a whole SIMD's registers for one wave, and one
-// wave cannot overlap its own MFMA and VALU work; so there are two passes that fit two
-// waves per SIMD:
-//   pass DK (DK = true):   S = A K1^T, dP = B V1^T, dS = P (dP - delta),  dK1^T += A^T dS
-//   pass DV (DK = false):  S = A K1^T,                                     dV1^T += B^T P
+// accumulators, K1 and V1 fragments) at D = 128 needs a whole SIMD's registers for one wave,
+// and one wave cannot overlap its own MFMA and VALU work; so at D = 128 there are two passes
+// that fit two waves per SIMD, and at D = 64 one kernel that does both:
+//   MODE kKvDk:    S = A K1^T, dP = B V1^T, dS = P (dP - delta),  dK1^T += A^T dS
+//   MODE kKvDv:    S = A K1^T,                                     dV1^T += B^T P
+//   MODE kKvBoth:  everything above from one S, one dP and one set of exponentials
 // with P = exp2(S scale log2e - lse).  Row-major tiles feed S and dP, copies with the
 // pitch of the transposed reads feed the accumulating products.  The two groups of a
 // slab hold partial sums that are added once, through LDS, at the end.
@@ -23,18 +24,24 @@
 
 namespace sa2 {
 
-template <int D, bool DK>
+constexpr int kKvDv = 0, kKvDk = 1, kKvBoth = 2;
+
+template <int D, int MODE>
 struct Kv8Cfg {
+    static constexpr bool DK = MODE != kKvDv;         // dK1 is produced (needs dP, delta, V1)
+    static constexpr bool DV = MODE != kKvDk;         // dV1 is produced
     static constexpr int PITCH = tile_pitch<D>();
     static constexpr int TILE = 32 * PITCH;
     static constexpr int TPITCH = tr_pitch<D>();
     static constexpr int TRT = 32 * TPITCH;
-    // step buffer: DK: [A row-major][A transposed-read copy][B row-major][lse][delta]
-    //              DV: [A row-major][B transposed-read][lse]
+    // step buffer: dk1:  [A row-major][A transposed-read copy][B row-major][lse][delta]
+    //              dv1:  [A row-major][B transposed-read][lse]
+    //              both: [A row-major][A transposed-read copy][B row-major][B transposed-read][lse][delta]
     static constexpr int AS = 0;
-    static constexpr int TR = TILE;                   // the tile read through transposed reads
-    static constexpr int BS = TILE + TRT;             // DK only
-    static constexpr int LSE = DK ? 2 * TILE + TRT : TILE + TRT;
+    static constexpr int ATR = TILE;                  // with dk1
+    static constexpr int BS = TILE + TRT;             // with dk1
+    static constexpr int BTR = DK ? 2 * TILE + TRT : TILE;   // with dv1
+    static constexpr int LSE = (DK ? 2 * TILE + TRT : TILE) + (DV ? TRT : 0);
     static constexpr int DEL = LSE + 32 * 4;
     static constexpr int STEP = DEL + 32 * 4;
     static constexpr int PAIR = 2 * STEP;
@@ -53,13 +60,16 @@ struct Kv8Cfg {
     static constexpr int RPT = (NROWP + 511) / 512;                 // ... per thread
     static constexpr int RPITCH = D + 4;              // floats per row of the final reduction
     static constexpr int LPT = 32 * D / 8 / 256;      // 16-byte pieces per thread and tensor
-    static_assert(128 * RPITCH * 4 <= TILES, "final reduction must fit the tile buffers");
+    static constexpr int RED = 128 * RPITCH * 4;      // bytes of one output's final reduction
+    static_assert((DK && DV ? 2 : 1) * RED <= TILES, "final reduction must fit the tile buffers");
 };
 
-template <int D, bool DK>
+template <int D, int MODE>
 __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     constexpr int KS = D / 16, DT = D / 32, PPR = D / 8;
-    using L = Kv8Cfg<D, DK>;
+    using L = Kv8Cfg<D, MODE>;
+    constexpr bool DK = L::DK, DV = L::DV, TWO = DK && DV;
+    static_assert(!TWO || D == 64, "both accumulators fit two waves per SIMD at D = 64 only");
     constexpr int PITCH = L::PITCH;
     __shared__ __attribute__((aligned(16))) char lds[L::LDS];
 
@@ -94,9 +104,12 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
             if constexpr (DK) v1f[kk] = ld_global16(v1row + (16 * kk + 8 * hf) * 2);
         }
     }
-    f32x16 acc[DT];
+    f32x16 acc[DT];              // dK1 (dV1 in the dv1-only pass)
+    f32x16 acc2[TWO ? DT : 1];   // dV1 when both are produced
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) acc[dt] = zero16();
+#pragma unroll
+    for (int dt = 0; dt < (TWO ? DT : 1); ++dt) acc2[dt] = zero16();
 #ifdef SA2_TIMING
     long long t_acc[6] = {0, 0, 0, 0, 0, 0};
     long long t_last = __builtin_amdgcn_s_memtime();
@@ -120,7 +133,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     const int wit_hi = ((jw + 31 + p.w1 - 1 < N - 1) ? jw + 31 + p.w1 - 1 : N - 1) / 32;
     const float c2 = p.scale_log2e;
     const int r_lane = c * PITCH + 16 * hf;
-    const int t_lane = L::TR + tr_lane_off<D, L::TPITCH>(lane);
+    const int t_lane = tr_lane_off<D, L::TPITCH>(lane);
 
     // ---- pair iterator (g, it, m): offsets 2m and 2m+1 of query tile `it`, query head g of the group
     struct Pair {
@@ -194,7 +207,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     // tile (the dk1 pass has no registers to spare and unpacks them once per pair)
     constexpr int PIECES = 32 * PPR;
     constexpr bool BOTH = PIECES == 512;
-    constexpr bool KEEP = !DK && BOTH;
+    constexpr bool KEEP = MODE == kKvDv && BOTH;
     const int b_row = (tid % PIECES) / PPR, b_col = (tid % PPR) * 16;
     float qx[8], ox[8];
     auto unpack_own = [&]() {
@@ -226,14 +239,14 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                 r0[w] = pack_bf16(xv[2 * w] * bf16_lo(f0[w]), xv[2 * w + 1] * bf16_hi(f0[w]));
                 r1[w] = pack_bf16(xv[2 * w] * bf16_lo(f1[w]), xv[2 * w + 1] * bf16_hi(f1[w]));
             }
-            // A: row-major (+ transposed-read copy in the dk1 pass); B: row-major in the dk1 pass, transposed-read in the dv1 pass
+            // A: row-major (+ transposed-read copy for dk1); B: row-major for dk1, transposed-read for dv1
             if (IS_A || DK) {
                 const int o = (IS_A ? L::AS : L::BS) + row * PITCH + col;
                 *reinterpret_cast<u32x4 *>(stage + o) = r0;
                 *reinterpret_cast<u32x4 *>(stage + L::STEP + o) = r1;
             }
-            if (IS_A == DK) {
-                const int o = L::TR + row * L::TPITCH + col;
+            if (IS_A ? DK : DV) {
+                const int o = (IS_A ? L::ATR : L::BTR) + row * L::TPITCH + col;
                 *reinterpret_cast<u32x4 *>(stage + o) = r0;
                 *reinterpret_cast<u32x4 *>(stage + L::STEP + o) = r1;
             }
@@ -350,11 +363,13 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                 X[rr] = ok ? X[rr] : -INFINITY;
             }
         }
-        u32x4 pb[2];
+        u32x4 pb[2];                 // dS with dk1, else P
+        u32x4 pv[TWO ? 2 : 1];       // P when both are produced
 #pragma unroll
         for (int rr = 0; rr < 16; rr += 2) {
             float p0 = fast_exp2(X[rr]);
             float p1 = fast_exp2(X[rr + 1]);
+            if constexpr (TWO) pv[rr >> 3][(rr & 7) >> 1] = pack_bf16(p0, p1);
             if constexpr (DK) {
                 p0 *= dP[rr];
                 p1 *= dP[rr + 1];
@@ -362,14 +377,17 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
             pb[rr >> 3][(rr & 7) >> 1] = pack_bf16(p0, p1);
         }
         TS(4);
+        auto tr_frag = [&](int image, int k2s, int dt) {
+            u32x2 lo2 = lds_read_tr<D, L::TPITCH>(buf + image + t_lane, 16 * k2s, 32 * dt);
+            u32x2 hi2 = lds_read_tr<D, L::TPITCH>(buf + image + t_lane, 16 * k2s + 8, 32 * dt);
+            return (u32x4){lo2[0], lo2[1], hi2[0], hi2[1]};
+        };
 #pragma unroll
         for (int k2s = 0; k2s < 2; ++k2s)
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
-                u32x2 lo2 = lds_read_tr<D, L::TPITCH>(buf + t_lane, 16 * k2s, 32 * dt);
-                u32x2 hi2 = lds_read_tr<D, L::TPITCH>(buf + t_lane, 16 * k2s + 8, 32 * dt);
-                u32x4 fr = {lo2[0], lo2[1], hi2[0], hi2[1]};
-                acc[dt] = mfma32(fr, pb[k2s], acc[dt]);
+                acc[dt] = mfma32(tr_frag(DK ? L::ATR : L::BTR, k2s, dt), pb[k2s], acc[dt]);
+                if constexpr (TWO) acc2[dt] = mfma32(tr_frag(L::BTR, k2s, dt), pv[k2s], acc2[dt]);
             }
         TS(5);
     }
@@ -385,30 +403,41 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     // ---- add the two groups of every slab and store
     __syncthreads();
     float *red = reinterpret_cast<float *>(lds) + (32 * slab + c) * L::RPITCH + 16 * hf;
-    if (pg == 1) {
+    auto publish = [&](const f32x16 (&a)[DT], float *dst) {
 #pragma unroll
         for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
             for (int r4 = 0; r4 < 4; ++r4)
-                *reinterpret_cast<float4 *>(red + 32 * dt + 4 * r4) =
-                    make_float4(acc[dt][4 * r4], acc[dt][4 * r4 + 1], acc[dt][4 * r4 + 2], acc[dt][4 * r4 + 3]);
+                *reinterpret_cast<float4 *>(dst + 32 * dt + 4 * r4) =
+                    make_float4(a[dt][4 * r4], a[dt][4 * r4 + 1], a[dt][4 * r4 + 2], a[dt][4 * r4 + 3]);
+    };
+    auto collect = [&](f32x16 (&a)[DT], const float *src) {
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+            for (int r4 = 0; r4 < 4; ++r4) {
+                const float4 v = *reinterpret_cast<const float4 *>(src + 32 * dt + 4 * r4);
+                a[dt][4 * r4] += v.x;
+                a[dt][4 * r4 + 1] += v.y;
+                a[dt][4 * r4 + 2] += v.z;
+                a[dt][4 * r4 + 3] += v.w;
+            }
+    };
+    if (pg == 1) {
+        publish(acc, red);
+        if constexpr (TWO) publish(acc2, red + L::RED / 4);
     }
     __syncthreads();
     if (pg == 1 || !j_ok) return;
-#pragma unroll
-    for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4) {
-            const float4 a = *reinterpret_cast<const float4 *>(red + 32 * dt + 4 * r4);
-            acc[dt][4 * r4] += a.x;
-            acc[dt][4 * r4 + 1] += a.y;
-            acc[dt][4 * r4 + 2] += a.z;
-            acc[dt][4 * r4 + 3] += a.w;
-        }
-    if constexpr (DK)
-        store_row<DT>(p.dk1.ptr + b * p.dk1.sb + (int64_t)j * p.dk1.sn + hk * p.dk1.sh + 16 * hf * 2, acc, p.scale);
-    else
-        store_row<DT>(p.dv1.ptr + b * p.dv1.sb + (int64_t)j * p.dv1.sn + hk * p.dv1.sh + 16 * hf * 2, acc, 1.f);
+    collect(acc, red);
+    char *dk1row = p.dk1.ptr + b * p.dk1.sb + (int64_t)j * p.dk1.sn + hk * p.dk1.sh + 16 * hf * 2;
+    char *dv1row = p.dv1.ptr + b * p.dv1.sb + (int64_t)j * p.dv1.sn + hk * p.dv1.sh + 16 * hf * 2;
+    if constexpr (DK) store_row<DT>(dk1row, acc, p.scale);
+    if constexpr (MODE == kKvDv) store_row<DT>(dv1row, acc, 1.f);
+    if constexpr (TWO) {
+        collect(acc2, red + L::RED / 4);
+        store_row<DT>(dv1row, acc2, 1.f);
+    }
 }
 
 }  // namespace sa2
