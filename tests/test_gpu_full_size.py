@@ -4,6 +4,7 @@ The CPU oracle cannot cover all (batch, head) slices of these shapes in test tim
   * one complete (batch, head) slice of config 3 is checked against the banded fp32 oracle
     (forward and all five gradients, all 8192 rows), and the other slices through batch /
     head independence: permuting the slices of the inputs permutes the outputs bit for bit;
+  * the layer shape of config 5 (grouped heads, dim_head 64) the same way;
   * config 4 (N = 32768) is checked through translation equivariance of the windows: the
     last rows of the full sequence must equal a run on the cropped sequence that still
     holds every row those queries can reach.
@@ -46,6 +47,31 @@ def test_config3_one_slice_against_oracle_and_slice_independence():
     assert torch.equal(flip(out_f), out)
     for a, b_ in zip(grads_f, grads):
         assert torch.equal(flip(a), b_)
+
+
+def test_config5_layer_one_group_against_oracle_and_slice_independence():
+    """Shape of one simplicial layer of config 5: B=8, N=2048, 8 query heads on 4 key/value
+    heads, dim_head 64 (at this head size dK1 and dV1 come from one kernel).  One batch entry
+    and one key/value head with its two query heads against the oracle, the rest through
+    batch / head independence."""
+    b, n, hq, hk, d, w1, w2 = 8, 2048, 8, 4, 64, 512, 32
+    ins = U.make_inputs(b, n, hq, hk, d, seed=4, std=d ** -0.5)
+    dev = [t.cuda() for t in ins]
+    out, grads = _run(*dev, w1, w2)
+    sb, sk = 5, 2
+    cut_q = lambda t: t[sb:sb + 1, :, 2 * sk:2 * sk + 2].contiguous()
+    cut_k = lambda t: t[sb:sb + 1, :, sk:sk + 1].contiguous()
+    q, k1, k2, v1, v2, dout = ins
+    ref_out, _, ref_grads = U.oracle_fwd_bwd(cut_q(q), cut_k(k1), cut_k(k2), cut_k(v1), cut_k(v2), cut_q(dout), w1, w2)
+    U.check_all(cut_q(out.cpu()), [cut_q(grads[0].cpu())] + [cut_k(t.cpu()) for t in grads[1:]], ref_out, ref_grads)
+    # reversing the batch order and the order of the key/value heads (query heads move with their group)
+    flip_k = lambda t: t.flip(0).flip(2).contiguous()
+    flip_q = lambda t: t.flip(0).unflatten(2, (hk, hq // hk)).flip(2).flatten(2, 3).contiguous()
+    flips = (flip_q, flip_k, flip_k, flip_k, flip_k, flip_q)
+    out_f, grads_f = _run(*(f(t) for f, t in zip(flips, dev)), w1, w2)
+    assert torch.equal(flip_q(out_f), out)
+    for f, a, b_ in zip(flips[:5], grads_f, grads):
+        assert torch.equal(f(a), b_)
 
 
 def test_config4_translation_equivariance():
