@@ -281,7 +281,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
             const bool valid = dlt <= dmax && i < N && i - dlt >= 0;
             char *st = stage + e * L::STEP;
             reinterpret_cast<float *>(st + L::LSE)[r] = valid ? reinterpret_cast<const float *>(lds + L::LSES)[r] : INFINITY;
-            if constexpr (DK) reinterpret_cast<float *>(st + L::DEL)[r] = valid ? reinterpret_cast<const float *>(lds + L::LSES)[32 + r] : 0.f;
+            if constexpr (DK) reinterpret_cast<float *>(st + L::DEL)[r] = valid ? -reinterpret_cast<const float *>(lds + L::LSES)[32 + r] : 0.f;
         }
     };
     auto next_tile = [&](Pair &s) {      // first pair of the next (query head, query tile)
@@ -334,7 +334,15 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
         f32x16 dP;
         if constexpr (DK) {
             __builtin_amdgcn_sched_barrier(0);        // keeps the two sets of fragments from being live together
-            dP = zero16();
+            // the accumulator starts at -delta_i (stored negated by the build): dP - delta costs no VALU work
+#pragma unroll
+            for (int a4 = 0; a4 < 4; ++a4) {
+                const float4 d4 = *reinterpret_cast<const float4 *>(buf + L::DEL + (8 * a4 + 4 * hf) * 4);
+                dP[4 * a4] = d4.x;
+                dP[4 * a4 + 1] = d4.y;
+                dP[4 * a4 + 2] = d4.z;
+                dP[4 * a4 + 3] = d4.w;
+            }
 #pragma unroll
             for (int kk = 0; kk < KS; ++kk) dP = mfma32(ld_lds16(buf + L::BS + r_lane + 32 * kk), v1f[kk], dP);
         }
@@ -345,13 +353,6 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
             X[4 * a4 + 1] = X[4 * a4 + 1] * c2 - l4.y;
             X[4 * a4 + 2] = X[4 * a4 + 2] * c2 - l4.z;
             X[4 * a4 + 3] = X[4 * a4 + 3] * c2 - l4.w;
-            if constexpr (DK) {
-                const float4 d4 = *reinterpret_cast<const float4 *>(buf + L::DEL + (8 * a4 + 4 * hf) * 4);
-                dP[4 * a4] -= d4.x;
-                dP[4 * a4 + 1] -= d4.y;
-                dP[4 * a4 + 2] -= d4.z;
-                dP[4 * a4 + 3] -= d4.w;
-            }
         }
         TS(3);
         const bool full = (jw + 31 <= 32 * it) && (jw + p.w1 > 32 * it + 31);
