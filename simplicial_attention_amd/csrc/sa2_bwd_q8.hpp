@@ -194,6 +194,9 @@ __global__ __launch_bounds__(512) void bwd_q8_kernel(KParams p, float *ws) {
     if (U > 1) issue_loads();
     int u = 0;
 
+    f32x16 neg_delta;          // DQ: -delta_i in every element (one query row per lane column)
+#pragma unroll
+    for (int rr = 0; rr < 16; ++rr) neg_delta[rr] = -dl;
     f32x16 acc[DT];            // G^T (DQ) or T^T (DV) of the running offset
     u32x4 A[KS];
     u32x4 Bv[DQ ? KS : 1];
@@ -240,9 +243,10 @@ __global__ __launch_bounds__(512) void bwd_q8_kernel(KParams p, float *ws) {
             for (int kk = 0; kk < KS; ++kk) X = mfma32(ld_lds16(sub + r_lane + 32 * kk), A[kk], X);
             f32x16 dP;
             if constexpr (DQ) {
-                dP = zero16();
+                // the chain starts from a register set that holds -delta_i: dP - delta costs no VALU work
+                dP = mfma32(ld_lds16(sub + C::OFF_V + r_lane), Bv[0], neg_delta);
 #pragma unroll
-                for (int kk = 0; kk < KS; ++kk) dP = mfma32(ld_lds16(sub + C::OFF_V + r_lane + 32 * kk), Bv[kk], dP);
+                for (int kk = 1; kk < KS; ++kk) dP = mfma32(ld_lds16(sub + C::OFF_V + r_lane + 32 * kk), Bv[kk], dP);
             }
 #pragma unroll
             for (int rr = 0; rr < 16; ++rr) X[rr] = X[rr] * c2 - lse2;
@@ -262,8 +266,8 @@ __global__ __launch_bounds__(512) void bwd_q8_kernel(KParams p, float *ws) {
                 float p0 = fast_exp2(X[rr]);
                 float p1 = fast_exp2(X[rr + 1]);
                 if constexpr (DQ) {
-                    p0 *= dP[rr] - dl;
-                    p1 *= dP[rr + 1] - dl;
+                    p0 *= dP[rr];
+                    p1 *= dP[rr + 1];
                 }
                 pb[rr >> 3][(rr & 7) >> 1] = pack_bf16(p0, p1);
             }
