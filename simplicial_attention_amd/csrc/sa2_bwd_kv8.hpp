@@ -12,9 +12,15 @@
 //   MODE kKvDk:    S = A K1^T, dP = B V1^T, dS = P (dP - delta),  dK1^T += A^T dS
 //   MODE kKvDv:    S = A K1^T,                                     dV1^T += B^T P
 //   MODE kKvBoth:  everything above from one S, one dP and one set of exponentials
-// with P = exp2(S scale log2e - lse).  Row-major tiles feed S and dP, copies with the
-// pitch of the transposed reads feed the accumulating products.  The two groups of a
-// slab hold partial sums that are added once, through LDS, at the end.
+// with P = exp2(S scale log2e - lse).  S and dP read row fragments of the A and B tiles
+// (ds_read_b128), the accumulating products read transposed fragments (ds_read_b64_tr_b16).
+// A tile that is read both ways is stored once, with the pitch of the transposed reads
+// (row starts 64 bytes apart modulo 256) and its 16-byte pieces XOR-swizzled inside every
+// aligned group of four: piece p of row r sits at piece p ^ ((r >> 2) & 3).  Transposed
+// reads touch whole 64-byte groups, so they stay conflict-free, and the sixteen rows a row
+// fragment read touches then cover all 64 banks.  LDS writes are the slow direction on
+// this chip (about 75 B/clk against 165 B/clk for reads), so one copy less is worth it.
+// The two groups of a slab hold partial sums that are added once, through LDS, at the end.
 #pragma once
 
 #include <type_traits>
@@ -34,14 +40,16 @@ struct Kv8Cfg {
     static constexpr int TILE = 32 * PITCH;
     static constexpr int TPITCH = tr_pitch<D>();
     static constexpr int TRT = 32 * TPITCH;
-    // step buffer: dk1:  [A row-major][A transposed-read copy][B row-major][lse][delta]
+    // step buffer: dk1:  [A swizzled][B row-major][lse][delta]
     //              dv1:  [A row-major][B transposed-read][lse]
-    //              both: [A row-major][A transposed-read copy][B row-major][B transposed-read][lse][delta]
+    //              both: [A swizzled][B swizzled][lse][delta]
+    static constexpr bool A_SWZ = DK;                 // A is read both ways
+    static constexpr bool B_SWZ = DK && DV;           // B is read both ways
+    static constexpr int A_PITCH = A_SWZ ? TPITCH : PITCH;
+    static constexpr int B_PITCH = DV ? TPITCH : PITCH;
     static constexpr int AS = 0;
-    static constexpr int ATR = TILE;                  // with dk1
-    static constexpr int BS = TILE + TRT;             // with dk1
-    static constexpr int BTR = DK ? 2 * TILE + TRT : TILE;   // with dv1
-    static constexpr int LSE = (DK ? 2 * TILE + TRT : TILE) + (DV ? TRT : 0);
+    static constexpr int BS = 32 * A_PITCH;
+    static constexpr int LSE = BS + 32 * B_PITCH;
     static constexpr int DEL = LSE + 32 * 4;
     static constexpr int STEP = DEL + 32 * 4;
     static constexpr int PAIR = 2 * STEP;
@@ -61,7 +69,7 @@ struct Kv8Cfg {
     static constexpr int RPITCH = D + 4;              // floats per row of the final reduction
     static constexpr int LPT = 32 * D / 8 / 256;      // 16-byte pieces per thread and tensor
     static constexpr int RED = 128 * RPITCH * 4;      // bytes of one output's final reduction
-    static_assert((DK && DV ? 2 : 1) * RED <= TILES, "final reduction must fit the tile buffers");
+    static_assert((DK && DV ? 2 : 1) * RED <= LDS, "final reduction must fit (everything else is dead by then)");
 };
 
 template <int D, int MODE>
@@ -132,8 +140,31 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     const int wit_lo = jw / 32;
     const int wit_hi = ((jw + 31 + p.w1 - 1 < N - 1) ? jw + 31 + p.w1 - 1 : N - 1) / 32;
     const float c2 = p.scale_log2e;
+    // per-lane parts of the fragment addresses.  Row fragments: row c, pieces 2 kk + hf.
+    // Transposed fragments: the lane's 8-byte chunk of tr_lane_off.  Swizzled tiles: the low
+    // two bits of the piece index are XORed with (row >> 2) & 3, which for row fragments
+    // leaves one base for even kk and one for odd kk, and for transposed fragments one base
+    // for the row blocks 16 s and one for the row blocks 16 s + 8.
     const int r_lane = c * PITCH + 16 * hf;
+    const int sg = ((c >> 2) & 3) ^ hf;
+    const int rs_even = c * L::TPITCH + 16 * sg, rs_odd = c * L::TPITCH + 16 * (sg ^ 2);
     const int t_lane = tr_lane_off<D, L::TPITCH>(lane);
+    const int t_row = 4 * (lane >> 5) + ((lane & 15) >> 2);
+    const int t_piece = (2 * (lane & 1) + ((lane >> 4) & 1)) ^ (lane >> 5);
+    const int ts_0 = t_row * L::TPITCH + 16 * t_piece + 8 * ((lane & 3) >> 1);
+    const int ts_8 = t_row * L::TPITCH + 16 * (t_piece ^ 2) + 8 * ((lane & 3) >> 1);
+    auto row_frag = [&](const char *image, auto swz, int kk) {
+        if constexpr (decltype(swz)::value) return ld_lds16(image + ((kk & 1) ? rs_odd : rs_even) + 64 * (kk >> 1));
+        else return ld_lds16(image + r_lane + 32 * kk);
+    };
+    auto tr_frag = [&](const char *image, auto swz, int k2s, int dt) {
+        constexpr bool SWZ = decltype(swz)::value;
+        u32x2 lo2 = lds_read_tr<D, L::TPITCH>(image + (SWZ ? ts_0 : t_lane), 16 * k2s, 32 * dt);
+        u32x2 hi2 = lds_read_tr<D, L::TPITCH>(image + (SWZ ? ts_8 : t_lane), 16 * k2s + 8, 32 * dt);
+        return (u32x4){lo2[0], lo2[1], hi2[0], hi2[1]};
+    };
+    using ASwz = std::integral_constant<bool, L::A_SWZ>;
+    using BSwz = std::integral_constant<bool, L::B_SWZ>;
 
     // ---- pair iterator (g, it, m): offsets 2m and 2m+1 of query tile `it`, query head g of the group
     struct Pair {
@@ -239,17 +270,11 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                 r0[w] = pack_bf16(xv[2 * w] * bf16_lo(f0[w]), xv[2 * w + 1] * bf16_hi(f0[w]));
                 r1[w] = pack_bf16(xv[2 * w] * bf16_lo(f1[w]), xv[2 * w + 1] * bf16_hi(f1[w]));
             }
-            // A: row-major (+ transposed-read copy for dk1); B: row-major for dk1, transposed-read for dv1
-            if (IS_A || DK) {
-                const int o = (IS_A ? L::AS : L::BS) + row * PITCH + col;
-                *reinterpret_cast<u32x4 *>(stage + o) = r0;
-                *reinterpret_cast<u32x4 *>(stage + L::STEP + o) = r1;
-            }
-            if (IS_A ? DK : DV) {
-                const int o = (IS_A ? L::ATR : L::BTR) + row * L::TPITCH + col;
-                *reinterpret_cast<u32x4 *>(stage + o) = r0;
-                *reinterpret_cast<u32x4 *>(stage + L::STEP + o) = r1;
-            }
+            constexpr bool SWZ = IS_A ? L::A_SWZ : L::B_SWZ;
+            const int pcol = SWZ ? (col ^ (((row >> 2) & 3) << 4)) : col;
+            const int o = (IS_A ? L::AS + row * L::A_PITCH : L::BS + row * L::B_PITCH) + pcol;
+            *reinterpret_cast<u32x4 *>(stage + o) = r0;
+            *reinterpret_cast<u32x4 *>(stage + L::STEP + o) = r1;
         };
         if constexpr (KEEP) {
             product(qx, L::K2S, std::true_type{});
@@ -330,7 +355,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
         // ---- S[i,j] (and dP[i,j]): rows = query rows of the tile, column = j
         f32x16 X = zero16();
 #pragma unroll
-        for (int kk = 0; kk < KS; ++kk) X = mfma32(ld_lds16(buf + L::AS + r_lane + 32 * kk), k1f[kk], X);
+        for (int kk = 0; kk < KS; ++kk) X = mfma32(row_frag(buf + L::AS, ASwz{}, kk), k1f[kk], X);
         f32x16 dP;
         if constexpr (DK) {
             __builtin_amdgcn_sched_barrier(0);        // keeps the two sets of fragments from being live together
@@ -344,7 +369,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                 dP[4 * a4 + 3] = d4.w;
             }
 #pragma unroll
-            for (int kk = 0; kk < KS; ++kk) dP = mfma32(ld_lds16(buf + L::BS + r_lane + 32 * kk), v1f[kk], dP);
+            for (int kk = 0; kk < KS; ++kk) dP = mfma32(row_frag(buf + L::BS, BSwz{}, kk), v1f[kk], dP);
         }
 #pragma unroll
         for (int a4 = 0; a4 < 4; ++a4) {
@@ -378,17 +403,13 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
             pb[rr >> 3][(rr & 7) >> 1] = pack_bf16(p0, p1);
         }
         TS(4);
-        auto tr_frag = [&](int image, int k2s, int dt) {
-            u32x2 lo2 = lds_read_tr<D, L::TPITCH>(buf + image + t_lane, 16 * k2s, 32 * dt);
-            u32x2 hi2 = lds_read_tr<D, L::TPITCH>(buf + image + t_lane, 16 * k2s + 8, 32 * dt);
-            return (u32x4){lo2[0], lo2[1], hi2[0], hi2[1]};
-        };
 #pragma unroll
         for (int k2s = 0; k2s < 2; ++k2s)
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) {
-                acc[dt] = mfma32(tr_frag(DK ? L::ATR : L::BTR, k2s, dt), pb[k2s], acc[dt]);
-                if constexpr (TWO) acc2[dt] = mfma32(tr_frag(L::BTR, k2s, dt), pv[k2s], acc2[dt]);
+                if constexpr (DK) acc[dt] = mfma32(tr_frag(buf + L::AS, ASwz{}, k2s, dt), pb[k2s], acc[dt]);
+                else acc[dt] = mfma32(tr_frag(buf + L::BS, BSwz{}, k2s, dt), pb[k2s], acc[dt]);
+                if constexpr (TWO) acc2[dt] = mfma32(tr_frag(buf + L::BS, BSwz{}, k2s, dt), pv[k2s], acc2[dt]);
             }
         TS(5);
     }
