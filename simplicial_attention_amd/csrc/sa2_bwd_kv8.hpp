@@ -14,12 +14,7 @@
 //   MODE kKvBoth:  everything above from one S, one dP and one set of exponentials
 // with P = exp2(S scale log2e - lse).  S and dP read row fragments of the A and B tiles
 // (ds_read_b128), the accumulating products read transposed fragments (ds_read_b64_tr_b16).
-// A tile that is read both ways is stored once, with the pitch of the transposed reads
-// (row starts 64 bytes apart modulo 256) and its 16-byte pieces XOR-swizzled inside every
-// aligned group of four: piece p of row r sits at piece p ^ ((r >> 2) & 3).  Transposed
-// reads touch whole 64-byte groups, so they stay conflict-free, and the sixteen rows a row
-// fragment read touches then cover all 64 banks.  LDS writes are the slow direction on
-// this chip (about 75 B/clk against 165 B/clk for reads), so one copy less is worth it.
+// A tile that is read both ways is stored once, in the swizzled layout of sa2_lds.hpp.
 // The two groups of a slab hold partial sums that are added once, through LDS, at the end.
 #pragma once
 
@@ -140,28 +135,22 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     const int wit_lo = jw / 32;
     const int wit_hi = ((jw + 31 + p.w1 - 1 < N - 1) ? jw + 31 + p.w1 - 1 : N - 1) / 32;
     const float c2 = p.scale_log2e;
-    // per-lane parts of the fragment addresses.  Row fragments: row c, pieces 2 kk + hf.
-    // Transposed fragments: the lane's 8-byte chunk of tr_lane_off.  Swizzled tiles: the low
-    // two bits of the piece index are XORed with (row >> 2) & 3, which for row fragments
-    // leaves one base for even kk and one for odd kk, and for transposed fragments one base
-    // for the row blocks 16 s and one for the row blocks 16 s + 8.
+    // per-lane parts of the fragment addresses: plain row-major / transposed-read tiles, swizzled tiles
     const int r_lane = c * PITCH + 16 * hf;
-    const int sg = ((c >> 2) & 3) ^ hf;
-    const int rs_even = c * L::TPITCH + 16 * sg, rs_odd = c * L::TPITCH + 16 * (sg ^ 2);
     const int t_lane = tr_lane_off<D, L::TPITCH>(lane);
-    const int t_row = 4 * (lane >> 5) + ((lane & 15) >> 2);
-    const int t_piece = (2 * (lane & 1) + ((lane >> 4) & 1)) ^ (lane >> 5);
-    const int ts_0 = t_row * L::TPITCH + 16 * t_piece + 8 * ((lane & 3) >> 1);
-    const int ts_8 = t_row * L::TPITCH + 16 * (t_piece ^ 2) + 8 * ((lane & 3) >> 1);
+    const SwzLane<D> swz_lane(lane);
     auto row_frag = [&](const char *image, auto swz, int kk) {
-        if constexpr (decltype(swz)::value) return ld_lds16(image + ((kk & 1) ? rs_odd : rs_even) + 64 * (kk >> 1));
+        if constexpr (decltype(swz)::value) return swz_lane.row_frag(image, kk);
         else return ld_lds16(image + r_lane + 32 * kk);
     };
     auto tr_frag = [&](const char *image, auto swz, int k2s, int dt) {
-        constexpr bool SWZ = decltype(swz)::value;
-        u32x2 lo2 = lds_read_tr<D, L::TPITCH>(image + (SWZ ? ts_0 : t_lane), 16 * k2s, 32 * dt);
-        u32x2 hi2 = lds_read_tr<D, L::TPITCH>(image + (SWZ ? ts_8 : t_lane), 16 * k2s + 8, 32 * dt);
-        return (u32x4){lo2[0], lo2[1], hi2[0], hi2[1]};
+        if constexpr (decltype(swz)::value) {
+            return swz_lane.tr_frag(image, k2s, dt);
+        } else {
+            const u32x2 lo2 = lds_read_tr<D, L::TPITCH>(image + t_lane, 16 * k2s, 32 * dt);
+            const u32x2 hi2 = lds_read_tr<D, L::TPITCH>(image + t_lane, 16 * k2s + 8, 32 * dt);
+            return (u32x4){lo2[0], lo2[1], hi2[0], hi2[1]};
+        }
     };
     using ASwz = std::integral_constant<bool, L::A_SWZ>;
     using BSwz = std::integral_constant<bool, L::B_SWZ>;
@@ -271,8 +260,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                 r1[w] = pack_bf16(xv[2 * w] * bf16_lo(f1[w]), xv[2 * w + 1] * bf16_hi(f1[w]));
             }
             constexpr bool SWZ = IS_A ? L::A_SWZ : L::B_SWZ;
-            const int pcol = SWZ ? (col ^ (((row >> 2) & 3) << 4)) : col;
-            const int o = (IS_A ? L::AS + row * L::A_PITCH : L::BS + row * L::B_PITCH) + pcol;
+            const int o = (IS_A ? L::AS : L::BS) + (SWZ ? swz_store_off<D>(row, col) : row * (IS_A ? L::A_PITCH : L::B_PITCH) + col);
             *reinterpret_cast<u32x4 *>(stage + o) = r0;
             *reinterpret_cast<u32x4 *>(stage + L::STEP + o) = r1;
         };

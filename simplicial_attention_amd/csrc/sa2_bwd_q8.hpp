@@ -38,10 +38,10 @@ struct Q8Cfg {
     static constexpr int TILE = 32 * PITCH;           // a tile read row-major
     static constexpr int TPITCH = tr_pitch<D>();
     static constexpr int TRT = 32 * TPITCH;           // a tile read through transposed reads
-    // sub-tile: DQ: [K1 row-major][K1 transposed-read copy][V1 row-major];  DV: [K1 row-major][V1 transposed-read]
-    static constexpr int OFF_TR = TILE;
-    static constexpr int OFF_V = TILE + TRT;          // DQ only
-    static constexpr int SUB = DQ ? 2 * TILE + TRT : TILE + TRT;
+    // sub-tile: DQ: [K1, read both ways: swizzled layout of sa2_lds.hpp][V1 row-major];  DV: [K1 row-major][V1 transposed-read]
+    static constexpr int OFF_TR = DQ ? 0 : TILE;      // the tile read through transposed reads
+    static constexpr int OFF_V = TRT;                 // DQ only
+    static constexpr int SUB = TILE + TRT;
     static constexpr int STAGE = CT * SUB;
     static constexpr int RING = 2 * STAGE;
     static constexpr int HALO = 31;
@@ -121,8 +121,8 @@ __global__ __launch_bounds__(512) void bwd_q8_kernel(KParams p, float *ws) {
     // ---- ring staging: the first PIECES threads move one 16-byte piece of K1 and of V1 per tile
     const bool stager = tid < C::PIECES;
     const int st_row = tid / PPR, st_col = (tid % PPR) * 16;
-    const int st_off = st_row * PITCH + st_col;
-    const int st_off_tr = C::OFF_TR + st_row * C::TPITCH + st_col;
+    const int st_off = DQ ? swz_store_off<D>(st_row, st_col) : st_row * PITCH + st_col;
+    const int st_off_tr = C::OFF_TR + st_row * C::TPITCH + st_col;                  // DV only
     const int st_off_v = C::OFF_V + st_row * PITCH + st_col;
     u32x4 st_k[CT], st_v[CT];
 #pragma unroll
@@ -150,7 +150,6 @@ __global__ __launch_bounds__(512) void bwd_q8_kernel(KParams p, float *ws) {
             for (int x = 0; x < CT; ++x) {
                 *reinterpret_cast<u32x4 *>(stage + x * C::SUB + st_off) = st_k[x];
                 if constexpr (DQ) {
-                    *reinterpret_cast<u32x4 *>(stage + x * C::SUB + st_off_tr) = st_k[x];
                     *reinterpret_cast<u32x4 *>(stage + x * C::SUB + st_off_v) = st_v[x];
                 } else {
                     *reinterpret_cast<u32x4 *>(stage + x * C::SUB + st_off_tr) = st_v[x];
@@ -160,6 +159,7 @@ __global__ __launch_bounds__(512) void bwd_q8_kernel(KParams p, float *ws) {
     };
     const int r_lane = c * PITCH + 16 * hf;                              // row-major fragment: row c, pieces 2*kk + hf
     const int t_lane = C::OFF_TR + tr_lane_off<D, C::TPITCH>(lane);      // transposed fragment, per-lane part
+    const SwzLane<D> swz_lane(lane);                                      // DQ: fragments of the swizzled K1 tile
 
     // ---- fp32 rows shared by the workgroup, zeroed; q/do/k2/v2 rows staged once
     float *dqs = reinterpret_cast<float *>(lds + C::DQS);
@@ -240,7 +240,7 @@ __global__ __launch_bounds__(512) void bwd_q8_kernel(KParams p, float *ws) {
             const char *sub = stage + x * C::SUB;
             f32x16 X = zero16();
 #pragma unroll
-            for (int kk = 0; kk < KS; ++kk) X = mfma32(ld_lds16(sub + r_lane + 32 * kk), A[kk], X);
+            for (int kk = 0; kk < KS; ++kk) X = mfma32(DQ ? swz_lane.row_frag(sub, kk) : ld_lds16(sub + r_lane + 32 * kk), A[kk], X);
             f32x16 dP;
             if constexpr (DQ) {
                 // the chain starts from a register set that holds -delta_i: dP - delta costs no VALU work
@@ -275,9 +275,14 @@ __global__ __launch_bounds__(512) void bwd_q8_kernel(KParams p, float *ws) {
             for (int k2s = 0; k2s < 2; ++k2s)
 #pragma unroll
                 for (int dt = 0; dt < DT; ++dt) {
-                    u32x2 lo = lds_read_tr<D, C::TPITCH>(sub + t_lane, 16 * k2s, 32 * dt);
-                    u32x2 hi = lds_read_tr<D, C::TPITCH>(sub + t_lane, 16 * k2s + 8, 32 * dt);
-                    u32x4 fr = {lo[0], lo[1], hi[0], hi[1]};
+                    u32x4 fr;
+                    if constexpr (DQ) {
+                        fr = swz_lane.tr_frag(sub, k2s, dt);
+                    } else {
+                        const u32x2 lo = lds_read_tr<D, C::TPITCH>(sub + t_lane, 16 * k2s, 32 * dt);
+                        const u32x2 hi = lds_read_tr<D, C::TPITCH>(sub + t_lane, 16 * k2s + 8, 32 * dt);
+                        fr = (u32x4){lo[0], lo[1], hi[0], hi[1]};
+                    }
                     acc[dt] = mfma32(fr, pb[k2s], acc[dt]);
                 }
         };

@@ -41,4 +41,47 @@ __device__ __forceinline__ u32x2 lds_read_tr(const char *lane_base, int row_base
     return __builtin_bit_cast(u32x2, v);
 }
 
+// A tile that is read both ways (row fragments with ds_read_b128 and transposed fragments
+// with ds_read_b64_tr_b16) is stored once: pitch tr_pitch (row starts 64 bytes apart
+// modulo 256) and the 16-byte pieces XOR-swizzled inside every aligned group of four,
+// piece p of row r at piece p ^ ((r >> 2) & 3).  Transposed reads touch whole 64-byte
+// groups, so the swizzle does not change their bank footprint; the sixteen rows that a
+// quarter of a row fragment read touches then cover all 64 banks.  One copy instead of two
+// matters because LDS writes are the slow direction on this chip (measured: about 75 B/clk
+// per CU against 165 B/clk for reads).
+template <int D>
+__device__ __forceinline__ int swz_store_off(int row, int byte_col) {
+    return row * tr_pitch<D>() + (byte_col ^ (((row >> 2) & 3) << 4));
+}
+
+// Per-lane parts of the fragment addresses of a swizzled tile.  Row fragment kk = row c,
+// pieces 2 kk + hf: the swizzle leaves one base for even kk and one for odd kk.  Transposed
+// fragment: the lane's 8-byte chunk of tr_lane_off, one base for the row blocks 16 s and
+// one for the row blocks 16 s + 8.
+template <int D>
+struct SwzLane {
+    static constexpr int P = tr_pitch<D>();
+    int rs_even, rs_odd, ts_0, ts_8;
+    __device__ __forceinline__ explicit SwzLane(int lane) {
+        const int c = lane & 31, hf = lane >> 5;
+        const int sg = ((c >> 2) & 3) ^ hf;
+        rs_even = c * P + 16 * sg;
+        rs_odd = c * P + 16 * (sg ^ 2);
+        const int row = 4 * (lane >> 5) + ((lane & 15) >> 2);
+        const int piece = (2 * (lane & 1) + ((lane >> 4) & 1)) ^ (lane >> 5);
+        ts_0 = row * P + 16 * piece + 8 * ((lane & 3) >> 1);
+        ts_8 = row * P + 16 * (piece ^ 2) + 8 * ((lane & 3) >> 1);
+    }
+    // row fragment kk (k-slots d = 16 kk + 8 hf .. + 7 of row c)
+    __device__ __forceinline__ u32x4 row_frag(const char *tile, int kk) const {
+        return ld_lds16(tile + ((kk & 1) ? rs_odd : rs_even) + 64 * (kk >> 1));
+    }
+    // transposed fragment: rows 16 k2s .. + 15 of the tile as k-slots, d tile dt as rows
+    __device__ __forceinline__ u32x4 tr_frag(const char *tile, int k2s, int dt) const {
+        const u32x2 lo = lds_read_tr<D, P>(tile + ts_0, 16 * k2s, 32 * dt);
+        const u32x2 hi = lds_read_tr<D, P>(tile + ts_8, 16 * k2s + 8, 32 * dt);
+        return (u32x4){lo[0], lo[1], hi[0], hi[1]};
+    }
+};
+
 }  // namespace sa2
