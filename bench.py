@@ -300,7 +300,7 @@ def main():
     # workload, scaled by what the same counters read for a 1 GiB device copy (profiles/pmc_cfg3_mfma_kernels.txt)
     measured_traffic = {
         'cfg3_raw_kernel_b4_h8_n8192_d128_w512_w32': {
-            'fwd': 2686022582, 'bwd_dq_dk2_pass': 742352823, 'bwd_dk1_pass': 646796522, 'bwd_dv1_pass': 514629355},
+            'fwd': 2686533563, 'bwd_dq_dk2_pass': 742062335, 'bwd_dk1_pass': 953681703, 'bwd_dv1_pass': 515353627},
     }
     traffic = measured_traffic.get(args.workload, {}).get(dom)
     roofline = {'bound': 'mfma', 'kernel': dom, 'kernel_symbol': symbols.get(dom), 'achieved': achieved, 'peak': PEAK_BF16_TFLOPS, 'unit': 'TFLOP/s',
