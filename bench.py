@@ -12,10 +12,10 @@ Algorithmic work (attended triples P per (batch, head), P = sum_i min(i+1,w1) mi
 `value` uses 18*D*B*H*P over the fwd+bwd time.  Each kernel is also timed on its own
 through the C ABI with HIP events on the launch stream; the `roofline` object is for
 the kernel with the longest launch, priced with the contractions that kernel needs
-for its own outputs (fwd 2: S, O; dQ/dK2 pass 3: S, dP, G; dV2 pass 2: S, T; dK1 pass 3:
-S, dP, dK1; dV1 pass 2: S, dV1; 2*D flop each per triple).  The backward entry points
-that launch two passes are also timed whole (4 contractions each: what their outputs
-need when S and dP are shared).
+for its own outputs (fwd 2: S, O; dQ/dK2 pass 3: S, dP, G; dV2 pass 2: S, T; dK1/dV1
+kernel 4: S, dP, dK1, dV1; 2*D flop each per triple).  The dQ/dK2/dV2 entry point, which
+launches several kernels, is also timed whole (4 contractions: what its outputs need when
+S and dP are shared).
 """
 import argparse
 import json
@@ -73,7 +73,7 @@ def main():
     ap.add_argument('--workload', default='cfg3_raw_kernel_b4_h8_n8192_d128_w512_w32', choices=sorted(WORKLOADS))
     ap.add_argument('--cpu-slices', type=int, default=4, help='(batch, head) slices of the CPU baseline sample (0 = skip)')
     ap.add_argument('--kernel-iters', type=int, default=5, help='launches per kernel for the per-kernel timing')
-    ap.add_argument('--only', default=None, help='time only this entry through the C ABI (fwd, bwd_delta, bwd_dq_dkv2, bwd_dkv1, bwd_dq_dk2_pass, bwd_dk1_pass, bwd_dv1_pass), `copy`: a 1 GiB device copy that calibrates HBM counters; `module_cfg2`: the module forward of config 2 and the fused qkv-norm kernel; `train_cfg5`: one training step of the config-5 language model; for profiling')
+    ap.add_argument('--only', default=None, help='time only this entry through the C ABI (fwd, bwd_delta, bwd_dq_dkv2, bwd_dkv1, bwd_dq_dk2_pass), `copy`: a 1 GiB device copy that calibrates HBM counters; `module_cfg2`: the module forward of config 2 and the fused qkv-norm kernel; `train_cfg5`: one training step of the config-5 language model; for profiling')
     args = ap.parse_args()
     if args.gpus != 1:
         print('bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path exists)', file=sys.stderr)
@@ -258,9 +258,7 @@ def main():
                     del os.environ['SA2_BWD_PASS']
             return run
         launches['bwd_dq_dk2_pass'] = (3, one_pass('first', launches['bwd_dq_dkv2'][1]))
-        if D == 128:         # at dim_head 64 one kernel produces dK1 and dV1 (bwd_dkv1 is a single launch)
-            launches['bwd_dk1_pass'] = (3, one_pass('first', launches['bwd_dkv1'][1]))
-            launches['bwd_dv1_pass'] = (2, one_pass('second', launches['bwd_dkv1'][1]))
+        # bwd_dkv1 is a single launch (one kernel produces dK1 and dV1)
     kernels = {}
     if args.only is not None:
         # the later kernels read what the earlier ones wrote: run the chain once, untimed
@@ -288,19 +286,18 @@ def main():
         return
     hbm_bytes = {'fwd': 7 * B * N * H * D * 2 + 4 * B * H * N, 'bwd_delta': 3 * B * N * H * D * 2 + 4 * B * H * N}
     # entries that are exactly one kernel launch (the two-pass entry points are timed per pass)
-    multi = () if w2 > 32 else ('bwd_dq_dkv2', 'bwd_dkv1') if D == 128 else ('bwd_dq_dkv2',)
+    multi = () if w2 > 32 else ('bwd_dq_dkv2',)
     single = [k for k in kernels if kernels[k]['contractions'] and k not in multi]
     dom = max(single, key=lambda k: kernels[k]['ms'])
     achieved = kernels[dom]['tflops']
-    symbols = {'fwd': 'sa2::fwd8_kernel<%d>' % D, 'bwd_dq_dk2_pass': 'sa2::bwd_q8_kernel<%d, true>' % D,
-               'bwd_dk1_pass': 'sa2::bwd_kv8_kernel<%d, 1>' % D, 'bwd_dv1_pass': 'sa2::bwd_kv8_kernel<%d, 0>' % D}
-    if D == 64 and w2 <= 32:
-        symbols['bwd_dkv1'] = 'sa2::bwd_kv8_kernel<64, 2>'
+    symbols = {'fwd': 'sa2::fwd8_kernel<%d>' % D, 'bwd_dq_dk2_pass': 'sa2::bwd_q8_kernel<%d, true>' % D}
+    if w2 <= 32:
+        symbols['bwd_dkv1'] = 'sa2::bwd_kv8_kernel<%d, %d>' % (D, 3 if D == 128 else 2)
     # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `--only <entry>` on this
     # workload, scaled by what the same counters read for a 1 GiB device copy (profiles/pmc_cfg3_mfma_kernels.txt)
     measured_traffic = {
         'cfg3_raw_kernel_b4_h8_n8192_d128_w512_w32': {
-            'fwd': 2686533563, 'bwd_dq_dk2_pass': 742062335, 'bwd_dk1_pass': 953681703, 'bwd_dv1_pass': 515353627},
+            'fwd': 2686533563, 'bwd_dq_dk2_pass': 742062335},
     }
     traffic = measured_traffic.get(args.workload, {}).get(dom)
     roofline = {'bound': 'mfma', 'kernel': dom, 'kernel_symbol': symbols.get(dom), 'achieved': achieved, 'peak': PEAK_BF16_TFLOPS, 'unit': 'TFLOP/s',

@@ -314,11 +314,15 @@ int sa2_bwd_dkv1(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor 
     const char *impl = std::getenv("SA2_BWD_KV1_IMPL");
     const bool fused = prob->w2 > 32 || (impl && std::strcmp(impl, "fused") == 0);
     const int pass = bwd_pass_filter();
+    const char *split = std::getenv("SA2_BWD_KV1_SPLIT");           // profiling knob: dK1 and dV1 in two passes
     if (!fused && prob->dim_head == 128) {
-        if (pass != 2) hipLaunchKernelGGL((sa2::bwd_kv8_kernel<128, sa2::kKvDk>), dim3(grid), dim3(512), 0, s, k);
-        if (pass != 1) hipLaunchKernelGGL((sa2::bwd_kv8_kernel<128, sa2::kKvDv>), dim3(grid), dim3(512), 0, s, k);
+        if (split && split[0] == '1') {
+            if (pass != 2) hipLaunchKernelGGL((sa2::bwd_kv8_kernel<128, sa2::kKvDk>), dim3(grid), dim3(512), 0, s, k);
+            if (pass != 1) hipLaunchKernelGGL((sa2::bwd_kv8_kernel<128, sa2::kKvDv>), dim3(grid), dim3(512), 0, s, k);
+        } else {
+            hipLaunchKernelGGL((sa2::bwd_kv8_kernel<128, sa2::kKvSplit>), dim3(grid), dim3(512), 0, s, k);
+        }
     } else if (!fused) {
-        const char *split = std::getenv("SA2_BWD_KV1_SPLIT");       // profiling knob: the two passes at dim_head 64 too
         if (split && split[0] == '1') {
             if (pass != 2) hipLaunchKernelGGL((sa2::bwd_kv8_kernel<64, sa2::kKvDk>), dim3(grid), dim3(512), 0, s, k);
             if (pass != 1) hipLaunchKernelGGL((sa2::bwd_kv8_kernel<64, sa2::kKvDv>), dim3(grid), dim3(512), 0, s, k);

@@ -12,6 +12,12 @@
 //   MODE kKvDk:    S = A K1^T, dP = B V1^T, dS = P (dP - delta),  dK1^T += A^T dS
 //   MODE kKvDv:    S = A K1^T,                                     dV1^T += B^T P
 //   MODE kKvBoth:  everything above from one S, one dP and one set of exponentials
+//   MODE kKvSplit: the same four contractions at D = 128, where one wave cannot hold both
+//                  accumulators: the two waves of a slab split the work instead of the
+//                  offsets.  Wave "P" forms S, P and dV1^T += B^T P for both offsets of the
+//                  pair and leaves the packed P in LDS; wave "S" forms dP meanwhile, then
+//                  (one barrier later) dS = P dP and dK1^T += A^T dS.  Two contractions per
+//                  wave and offset, one operand build per pair, no final reduction.
 // with P = exp2(S scale log2e - lse).  S and dP read row fragments of the A and B tiles
 // (ds_read_b128), the accumulating products read transposed fragments (ds_read_b64_tr_b16).
 // A tile that is read both ways is stored once, in the swizzled layout of sa2_lds.hpp.
@@ -25,7 +31,7 @@
 
 namespace sa2 {
 
-constexpr int kKvDv = 0, kKvDk = 1, kKvBoth = 2;
+constexpr int kKvDv = 0, kKvDk = 1, kKvBoth = 2, kKvSplit = 3;
 
 template <int D, int MODE>
 struct Kv8Cfg {
@@ -58,20 +64,21 @@ struct Kv8Cfg {
     static constexpr int K2S = DOS + 32 * RP;
     static constexpr int V2S = K2S + KROWS * RP;
     static constexpr int LSES = V2S + KROWS * RP;     // 32 floats lse * log2e, 32 floats delta
-    static constexpr int LDS = LSES + 64 * 4;
+    static constexpr int PX = LSES + 64 * 4;          // kKvSplit: packed P of [slab][offset of the pair], 2 KiB each
+    static constexpr int LDS = PX + (MODE == kKvSplit ? 4 * 2 * 2048 : 0);
     static constexpr int NROWP = (64 + 2 * KROWS) * (D / 8);        // 16-byte pieces of the staged rows
     static constexpr int RPT = (NROWP + 511) / 512;                 // ... per thread
     static constexpr int RPITCH = D + 4;              // floats per row of the final reduction
     static constexpr int LPT = 32 * D / 8 / 256;      // 16-byte pieces per thread and tensor
     static constexpr int RED = 128 * RPITCH * 4;      // bytes of one output's final reduction
-    static_assert((DK && DV ? 2 : 1) * RED <= LDS, "final reduction must fit (everything else is dead by then)");
+    static_assert((MODE == kKvBoth ? 2 : 1) * RED <= LDS, "final reduction must fit (everything else is dead by then)");
 };
 
 template <int D, int MODE>
 __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     constexpr int KS = D / 16, DT = D / 32, PPR = D / 8;
     using L = Kv8Cfg<D, MODE>;
-    constexpr bool DK = L::DK, DV = L::DV, TWO = DK && DV;
+    constexpr bool DK = L::DK, DV = L::DV, TWO = MODE == kKvBoth, SPLIT = MODE == kKvSplit;
     static_assert(!TWO || D == 64, "both accumulators fit two waves per SIMD at D = 64 only");
     constexpr int PITCH = L::PITCH;
     __shared__ __attribute__((aligned(16))) char lds[L::LDS];
@@ -96,15 +103,16 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     const char *k2g = p.k2.ptr + b * p.k2.sb + hk * p.k2.sh;
     const char *v2g = p.v2.ptr + b * p.v2.sb + hk * p.v2.sh;
 
-    u32x4 k1f[KS];
-    u32x4 v1f[DK ? KS : 1];
+    u32x4 k1f[KS];                        // kKvSplit: the K1 rows in the P waves, the V1 rows in the S waves
+    u32x4 v1f[(DK && !SPLIT) ? KS : 1];
     {
         const char *k1row = p.k1.ptr + b * p.k1.sb + (int64_t)jc * p.k1.sn + hk * p.k1.sh;
         const char *v1row = p.v1.ptr + b * p.v1.sb + (int64_t)jc * p.v1.sn + hk * p.v1.sh;
+        const char *own = (SPLIT && pg == 1) ? v1row : k1row;
 #pragma unroll
         for (int kk = 0; kk < KS; ++kk) {
-            k1f[kk] = ld_global16(k1row + (16 * kk + 8 * hf) * 2);
-            if constexpr (DK) v1f[kk] = ld_global16(v1row + (16 * kk + 8 * hf) * 2);
+            k1f[kk] = ld_global16(own + (16 * kk + 8 * hf) * 2);
+            if constexpr (DK && !SPLIT) v1f[kk] = ld_global16(v1row + (16 * kk + 8 * hf) * 2);
         }
     }
     f32x16 acc[DT];              // dK1 (dV1 in the dv1-only pass)
@@ -316,6 +324,130 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     if constexpr (KEEP) unpack_own();
     build(nb, 0);
     next_pair(nb);
+
+    if constexpr (SPLIT) {
+        // The two roles run separate loops with the same barrier sequence (per pair: tiles
+        // complete; [new query tile: rows replaced]; P in LDS), so that neither loop carries
+        // the other role's registers.
+        char *px = lds + L::PX + slab * 4096 + lane * 16;       // [offset of the pair][half] 1 KiB each
+        auto open_pair = [&](bool more) {
+            __syncthreads();                                    // the tiles of the pair are complete
+            if (more && nb.m == 0) {
+                write_rows();
+                next_tile(rw);
+                if (rw.g < p.G) issue_rows(rw);
+                __syncthreads();
+            }
+        };
+        if (pg == 0) {
+            // ---- P waves: S, P (left in LDS for the other wave of the slab), dV1^T += B^T P
+            for (int s = 0; s < npairs; ++s) {
+                const bool more = s + 1 < npairs;
+                open_pair(more);
+                const char *pair = lds + (s & 1) * L::PAIR;
+                const int it = cur.it;
+                next_pair(cur);
+                if (wave_active && it >= wit_lo && it <= wit_hi) {
+                    const bool full = (jw + 31 <= 32 * it) && (jw + p.w1 > 32 * it + 31);
+#pragma unroll
+                    for (int e = 0; e < 2; ++e) {
+                        const char *buf = pair + e * L::STEP;
+                        f32x16 X = zero16();
+#pragma unroll
+                        for (int kk = 0; kk < KS; ++kk) X = mfma32(swz_lane.row_frag(buf + L::AS, kk), k1f[kk], X);
+#pragma unroll
+                        for (int a4 = 0; a4 < 4; ++a4) {
+                            const float4 l4 = *reinterpret_cast<const float4 *>(buf + L::LSE + (8 * a4 + 4 * hf) * 4);
+                            X[4 * a4] = X[4 * a4] * c2 - l4.x;
+                            X[4 * a4 + 1] = X[4 * a4 + 1] * c2 - l4.y;
+                            X[4 * a4 + 2] = X[4 * a4 + 2] * c2 - l4.z;
+                            X[4 * a4 + 3] = X[4 * a4 + 3] * c2 - l4.w;
+                        }
+                        if (!full) {
+                            const int base = 32 * it + 4 * hf - j;   // i - j for register 0
+#pragma unroll
+                            for (int rr = 0; rr < 16; ++rr) {
+                                const bool ok = (unsigned)(base + 8 * (rr >> 2) + (rr & 3)) < (unsigned)p.w1;
+                                X[rr] = ok ? X[rr] : -INFINITY;
+                            }
+                        }
+                        u32x4 pb[2];
+#pragma unroll
+                        for (int rr = 0; rr < 16; rr += 2)
+                            pb[rr >> 3][(rr & 7) >> 1] = pack_bf16(fast_exp2(X[rr]), fast_exp2(X[rr + 1]));
+                        *reinterpret_cast<u32x4 *>(px + e * 2048) = pb[0];
+                        *reinterpret_cast<u32x4 *>(px + e * 2048 + 1024) = pb[1];
+#pragma unroll
+                        for (int k2s = 0; k2s < 2; ++k2s)
+#pragma unroll
+                            for (int dt = 0; dt < DT; ++dt) acc[dt] = mfma32(swz_lane.tr_frag(buf + L::BS, k2s, dt), pb[k2s], acc[dt]);
+                        __builtin_amdgcn_sched_barrier(0);      // one offset at a time: its fragments are dead before the next one's are loaded
+                    }
+                }
+                __syncthreads();                                // P of the pair is in LDS
+                if (more) {
+                    build(nb, (s + 1) & 1);                     // the P waves' share of the next pair's tiles
+                    next_pair(nb);
+                }
+            }
+            if (j_ok) store_row<DT>(p.dv1.ptr + b * p.dv1.sb + (int64_t)j * p.dv1.sn + hk * p.dv1.sh + 16 * hf * 2, acc, 1.f);
+        } else {
+            // ---- S waves: their share of the next pair's tiles, dP - delta for both offsets; after
+            // the barrier dS = P (dP - delta), dK1^T += A^T dS
+            for (int s = 0; s < npairs; ++s) {
+                const bool more = s + 1 < npairs;
+                open_pair(more);
+                const char *pair = lds + (s & 1) * L::PAIR;
+                const int it = cur.it;
+                next_pair(cur);
+                const bool on = wave_active && it >= wit_lo && it <= wit_hi;
+                if (more) {
+                    build(nb, (s + 1) & 1);
+                    next_pair(nb);
+                }
+                f32x16 dPe[2];
+                if (on) {
+#pragma unroll
+                    for (int e = 0; e < 2; ++e) {
+                        const char *buf = pair + e * L::STEP;
+#pragma unroll
+                        for (int a4 = 0; a4 < 4; ++a4) {
+                            const float4 d4 = *reinterpret_cast<const float4 *>(buf + L::DEL + (8 * a4 + 4 * hf) * 4);
+                            dPe[e][4 * a4] = d4.x;
+                            dPe[e][4 * a4 + 1] = d4.y;
+                            dPe[e][4 * a4 + 2] = d4.z;
+                            dPe[e][4 * a4 + 3] = d4.w;
+                        }
+#pragma unroll
+                        for (int kk = 0; kk < KS; ++kk) dPe[e] = mfma32(swz_lane.row_frag(buf + L::BS, kk), k1f[kk], dPe[e]);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+                __syncthreads();                                // P of the pair is in LDS
+                if (on) {
+#pragma unroll
+                    for (int e = 0; e < 2; ++e) {
+                        const char *buf = pair + e * L::STEP;
+                        u32x4 pb[2];
+#pragma unroll
+                        for (int hh = 0; hh < 2; ++hh) {
+                            const u32x4 pq = ld_lds16(px + e * 2048 + hh * 1024);
+#pragma unroll
+                            for (int w = 0; w < 4; ++w)
+                                pb[hh][w] = pack_bf16(bf16_lo(pq[w]) * dPe[e][8 * hh + 2 * w], bf16_hi(pq[w]) * dPe[e][8 * hh + 2 * w + 1]);
+                        }
+#pragma unroll
+                        for (int k2s = 0; k2s < 2; ++k2s)
+#pragma unroll
+                            for (int dt = 0; dt < DT; ++dt) acc[dt] = mfma32(swz_lane.tr_frag(buf + L::AS, k2s, dt), pb[k2s], acc[dt]);
+                        __builtin_amdgcn_sched_barrier(0);
+                    }
+                }
+            }
+            if (j_ok) store_row<DT>(p.dk1.ptr + b * p.dk1.sb + (int64_t)j * p.dk1.sn + hk * p.dk1.sh + 16 * hf * 2, acc, p.scale);
+        }
+        return;
+    }
 
     for (int s = 0; s < npairs; ++s) {
         __syncthreads();
