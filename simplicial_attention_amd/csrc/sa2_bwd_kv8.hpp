@@ -347,7 +347,9 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                 const char *pair = lds + (s & 1) * L::PAIR;
                 const int it = cur.it;
                 next_pair(cur);
-                if (wave_active && it >= wit_lo && it <= wit_hi) {
+                const bool on = wave_active && it >= wit_lo && it <= wit_hi;
+                u32x4 pb_late[2];                               // P of the second offset: its dV1 products run after the barrier
+                if (on) {
                     const bool full = (jw + 31 <= 32 * it) && (jw + p.w1 > 32 * it + 31);
 #pragma unroll
                     for (int e = 0; e < 2; ++e) {
@@ -377,14 +379,27 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                             pb[rr >> 3][(rr & 7) >> 1] = pack_bf16(fast_exp2(X[rr]), fast_exp2(X[rr + 1]));
                         *reinterpret_cast<u32x4 *>(px + e * 2048) = pb[0];
                         *reinterpret_cast<u32x4 *>(px + e * 2048 + 1024) = pb[1];
+                        if (e == 0) {
 #pragma unroll
-                        for (int k2s = 0; k2s < 2; ++k2s)
+                            for (int k2s = 0; k2s < 2; ++k2s)
 #pragma unroll
-                            for (int dt = 0; dt < DT; ++dt) acc[dt] = mfma32(swz_lane.tr_frag(buf + L::BS, k2s, dt), pb[k2s], acc[dt]);
+                                for (int dt = 0; dt < DT; ++dt) acc[dt] = mfma32(swz_lane.tr_frag(buf + L::BS, k2s, dt), pb[k2s], acc[dt]);
+                        } else {
+                            pb_late[0] = pb[0];
+                            pb_late[1] = pb[1];
+                        }
                         __builtin_amdgcn_sched_barrier(0);      // one offset at a time: its fragments are dead before the next one's are loaded
                     }
                 }
                 __syncthreads();                                // P of the pair is in LDS
+                if (on) {
+                    // the S waves now have MFMA and VALU work of their own; this evens out the two halves
+                    const char *buf = pair + L::STEP;
+#pragma unroll
+                    for (int k2s = 0; k2s < 2; ++k2s)
+#pragma unroll
+                        for (int dt = 0; dt < DT; ++dt) acc[dt] = mfma32(swz_lane.tr_frag(buf + L::BS, k2s, dt), pb_late[k2s], acc[dt]);
+                }
                 if (more) {
                     build(nb, (s + 1) & 1);                     // the P waves' share of the next pair's tiles
                     next_pair(nb);
