@@ -131,13 +131,15 @@ def test_other_head_dimensions_and_dtypes(dtype, dqk, dv, n, w1, w2):
     U.check_all(out, grads, ref_out, ref_grads, unit_variance=True)
 
 
-def test_dim_head_64_two_pass_key_value_backward(monkeypatch):
-    """SA2_BWD_KV1_SPLIT=1: dK1 and dV1 at dim_head 64 from the two passes that dim_head 128
-    uses, instead of the single kernel that produces both."""
+@pytest.mark.parametrize('shape', [(2, 200, 4, 2, 64, 64, 32), (1, 300, 2, 2, 128, 96, 16)])
+def test_two_pass_key_value_backward(shape, monkeypatch):
+    """SA2_BWD_KV1_SPLIT=1: dK1 and dV1 from two passes (each recomputing S) instead of the
+    single kernel that produces both."""
     monkeypatch.setenv('SA2_BWD_KV1_SPLIT', '1')
-    ins = U.make_inputs(2, 200, 4, 2, 64, seed=29, std=64 ** -0.5)
-    ref_out, _, ref_grads = U.oracle_fwd_bwd(*ins, 64, 32)
-    out, grads = U.hip_fwd_bwd(*ins, 64, 32)
+    b, n, hq, hk, d, w1, w2 = shape
+    ins = U.make_inputs(b, n, hq, hk, d, seed=29, std=d ** -0.5)
+    ref_out, _, ref_grads = U.oracle_fwd_bwd(*ins, w1, w2)
+    out, grads = U.hip_fwd_bwd(*ins, w1, w2)
     U.check_all(out, grads, ref_out, ref_grads)
 
 
