@@ -1,27 +1,31 @@
-// Backward kernels for dK1 and for dV1, eight-wave variant (two waves per SIMD).
+// Backward kernels for dK1 and dV1, eight-wave variant (two waves per SIMD).
 //
-// Workgroup = 128 rows j of one (batch, kv head).  The eight waves are four 32-row slabs
-// of j times two step groups: the workgroup walks pairs of "steps" (query head of the
-// group, 32-row query tile, offset dlt); of a pair, the waves of group 0 take the even
-// offset and the waves of group 1 the odd one.  The q/do rows of a query tile and the 63
-// k2/v2 rows its offsets (at most 32) can reach are staged in LDS once per tile; from
-// them the 512 threads build A = q*k2 and B = do*v2 of both steps once per barrier.  A fused kernel (dK1 and dV1
-// accumulators, K1 and V1 fragments) at D = 128 needs a whole SIMD's registers for one wave,
-// and one wave cannot overlap its own MFMA and VALU work; so at D = 128 there are two passes
-// that fit two waves per SIMD, and at D = 64 one kernel that does both:
-//   MODE kKvDk:    S = A K1^T, dP = B V1^T, dS = P (dP - delta),  dK1^T += A^T dS
-//   MODE kKvDv:    S = A K1^T,                                     dV1^T += B^T P
-//   MODE kKvBoth:  everything above from one S, one dP and one set of exponentials
-//   MODE kKvSplit: the same four contractions at D = 128, where one wave cannot hold both
-//                  accumulators: the two waves of a slab split the work instead of the
-//                  offsets.  Wave "P" forms S, P and dV1^T += B^T P for both offsets of the
-//                  pair and leaves the packed P in LDS; wave "S" forms dP meanwhile, then
-//                  (one barrier later) dS = P dP and dK1^T += A^T dS.  Two contractions per
-//                  wave and offset, one operand build per pair, no final reduction.
-// with P = exp2(S scale log2e - lse).  S and dP read row fragments of the A and B tiles
-// (ds_read_b128), the accumulating products read transposed fragments (ds_read_b64_tr_b16).
-// A tile that is read both ways is stored once, in the swizzled layout of sa2_lds.hpp.
-// The two groups of a slab hold partial sums that are added once, through LDS, at the end.
+// Workgroup = 128 rows j of one (batch, kv head): four 32-row slabs of j, two waves per
+// slab.  The workgroup walks pairs of "steps" (query head of the group, 32-row query tile,
+// offset dlt); a pair holds the offsets 2m and 2m+1 of one query tile.  The q/do rows of a
+// query tile and the 63 k2/v2 rows its offsets (at most 32) can reach are staged in LDS
+// once per tile; from them the 512 threads build A = q*k2 and B = do*v2 of both steps
+// once per pair.  With P = exp2(S scale log2e - lse):
+//   S = A K1^T,  dP = B V1^T,  dS = P (dP - delta),  dK1^T += A^T dS,  dV1^T += B^T P.
+// One wave cannot overlap its own MFMA and VALU work, so every variant keeps two waves per
+// SIMD (at most 256 registers per wave):
+//   MODE kKvBoth  (D = 64):  both accumulators fit one wave.  The two waves of a slab take
+//                  one offset of the pair each and form all four products from one S, one
+//                  dP and one set of exponentials; their partial sums are added once,
+//                  through LDS, at the end.
+//   MODE kKvSplit (D = 128): one wave cannot hold both accumulators, so the two waves of a
+//                  slab split the work instead of the offsets.  Wave "P" holds the K1 rows
+//                  and the dV1 accumulator: S, P and dV1^T += B^T P for both offsets of the
+//                  pair, and it leaves the packed P in LDS.  Wave "S" holds the V1 rows and
+//                  the dK1 accumulator: dP - delta meanwhile, then (one barrier later)
+//                  dS = P dP and dK1^T += A^T dS.  Two contractions per wave and offset,
+//                  one operand build per pair, no final reduction.
+//   MODE kKvDk / kKvDv:  two passes that each recompute S (dK1 with S, dP; dV1 with S);
+//                  offsets split between the two waves of a slab as in kKvBoth.  Kept as
+//                  a cross-check of the single-kernel variants.
+// S and dP read row fragments of the A and B tiles (ds_read_b128), the accumulating
+// products read transposed fragments (ds_read_b64_tr_b16).  A tile that is read both ways
+// is stored once, in the swizzled layout of sa2_lds.hpp.
 #pragma once
 
 #include <type_traits>
