@@ -149,10 +149,15 @@ int sa2_fwd(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, 
         k.m_save = saved->m;
     }
     const int grid = prob->batch * prob->heads * ((prob->seq_len + 31) / 32);
-    if (prob->dim_head == 128)
-        hipLaunchKernelGGL(sa2::fwd8_kernel<128>, dim3(grid), dim3(512), 0, s, k);
-    else
-        hipLaunchKernelGGL(sa2::fwd8_kernel<64>, dim3(grid), dim3(512), 0, s, k);
+    // the instance for second windows up to 32 stages fewer k2/v2 rows (at dim_head 64 two workgroups fit a CU)
+    const bool narrow = prob->w2 <= 32;
+    if (prob->dim_head == 128) {
+        if (narrow) hipLaunchKernelGGL((sa2::fwd8_kernel<128, 32>), dim3(grid), dim3(512), 0, s, k);
+        else hipLaunchKernelGGL((sa2::fwd8_kernel<128, 64>), dim3(grid), dim3(512), 0, s, k);
+    } else {
+        if (narrow) hipLaunchKernelGGL((sa2::fwd8_kernel<64, 32>), dim3(grid), dim3(512), 0, s, k);
+        else hipLaunchKernelGGL((sa2::fwd8_kernel<64, 64>), dim3(grid), dim3(512), 0, s, k);
+    }
     return after_launch("forward");
 }
 

@@ -29,7 +29,7 @@
 
 namespace sa2 {
 
-template <int D>
+template <int D, int W2MAX_>
 struct Fwd8 {
     static constexpr int KS = D / 16;
     static constexpr int DT = D / 32;
@@ -44,7 +44,7 @@ struct Fwd8 {
     static constexpr int APITCH = D + 4;              // floats per row of the shared accumulator
     static constexpr int ACC = 32 * APITCH * 4;
     static constexpr int EXCH = 8 * 32 * 4;           // one float per (wave, row)
-    static constexpr int W2MAX = 64;                  // largest second window the kernels accept
+    static constexpr int W2MAX = W2MAX_;              // largest second window this instance accepts (32 or 64)
     static constexpr int SROWS = 32 + W2MAX - 1;      // rows k in [i0-(W2MAX-1), i0+31]
     static constexpr int QS = RING + ACC + 2 * EXCH;  // q rows of the tile      [32][pitch]
     static constexpr int K2S = QS + TILE;             // k2 rows                 [SROWS][pitch]
@@ -53,9 +53,9 @@ struct Fwd8 {
     static constexpr int PIECES = 32 * D / 8;         // 16-byte pieces per tile
 };
 
-template <int D>
-__global__ __launch_bounds__(512) void fwd8_kernel(KParams p) {
-    using C = Fwd8<D>;
+template <int D, int W2MAX>
+__global__ __launch_bounds__(512, (D == 64 && W2MAX == 32) ? 4 : 1) void fwd8_kernel(KParams p) {
+    using C = Fwd8<D, W2MAX>;
     constexpr int KS = C::KS, DT = C::DT, CT = C::CT, PPR = D / 8, PITCH = tile_pitch<D>();
     __shared__ __attribute__((aligned(16))) char lds[C::LDS];
 
