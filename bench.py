@@ -290,14 +290,14 @@ def main():
     single = [k for k in kernels if kernels[k]['contractions'] and k not in multi]
     dom = max(single, key=lambda k: kernels[k]['ms'])
     achieved = kernels[dom]['tflops']
-    symbols = {'fwd': 'sa2::fwd8_kernel<%d>' % D, 'bwd_dq_dk2_pass': 'sa2::bwd_q8_kernel<%d, true>' % D}
+    symbols = {'fwd': 'sa2::fwd8_kernel<%d, %d>' % (D, 32 if w2 <= 32 else 64), 'bwd_dq_dk2_pass': 'sa2::bwd_q8_kernel<%d, true>' % D}
     if w2 <= 32:
         symbols['bwd_dkv1'] = 'sa2::bwd_kv8_kernel<%d, %d>' % (D, 3 if D == 128 else 2)
     # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `--only <entry>` on this
     # workload, scaled by what the same counters read for a 1 GiB device copy (profiles/pmc_cfg3_mfma_kernels.txt)
     measured_traffic = {
         'cfg3_raw_kernel_b4_h8_n8192_d128_w512_w32': {
-            'fwd': 2685857830, 'bwd_dq_dk2_pass': 742120219, 'bwd_dkv1': 724346796},
+            'fwd': 2673834064, 'bwd_dq_dk2_pass': 736323779, 'bwd_dkv1': 739411429},
     }
     traffic = measured_traffic.get(args.workload, {}).get(dom)
     roofline = {'bound': 'mfma', 'kernel': dom, 'kernel_symbol': symbols.get(dom), 'achieved': achieved, 'peak': PEAK_BF16_TFLOPS, 'unit': 'TFLOP/s',
