@@ -411,7 +411,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
             }
             if (j_ok) store_row<DT>(p.dv1.ptr + b * p.dv1.sb + (int64_t)j * p.dv1.sn + hk * p.dv1.sh + 16 * hf * 2, acc, 1.f);
         } else {
-            // ---- S waves: their share of the next pair's tiles, dP - delta for both offsets; after
+            // ---- S waves: dP - delta for both offsets, their share of the next pair's tiles; after
             // the barrier dS = P (dP - delta), dK1^T += A^T dS
             for (int s = 0; s < npairs; ++s) {
                 const bool more = s + 1 < npairs;
@@ -420,10 +420,6 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                 const int it = cur.it;
                 next_pair(cur);
                 const bool on = wave_active && it >= wit_lo && it <= wit_hi;
-                if (more) {
-                    build(nb, (s + 1) & 1);
-                    next_pair(nb);
-                }
                 f32x16 dPe[2];
                 if (on) {
 #pragma unroll
@@ -441,6 +437,12 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                         for (int kk = 0; kk < KS; ++kk) dPe[e] = mfma32(swz_lane.row_frag(buf + L::BS, kk), k1f[kk], dPe[e]);
                         __builtin_amdgcn_sched_barrier(0);
                     }
+                }
+                // the MFMA chains first, the build after them: measured faster than the other order
+                // (the P waves start the pair with MFMA work as well and then turn to their exponentials)
+                if (more) {
+                    build(nb, (s + 1) & 1);
+                    next_pair(nb);
                 }
                 __syncthreads();                                // P of the pair is in LDS
                 if (on) {
