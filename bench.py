@@ -297,7 +297,7 @@ def main():
     # workload, scaled by what the same counters read for a 1 GiB device copy (profiles/pmc_cfg3_mfma_kernels.txt)
     measured_traffic = {
         'cfg3_raw_kernel_b4_h8_n8192_d128_w512_w32': {
-            'fwd': 2673834064, 'bwd_dq_dk2_pass': 736323779, 'bwd_dkv1': 739411429},
+            'fwd': 2682106604, 'bwd_dq_dk2_pass': 736942192, 'bwd_dkv1': 710897605},
     }
     traffic = measured_traffic.get(args.workload, {}).get(dom)
     roofline = {'bound': 'mfma', 'kernel': dom, 'kernel_symbol': symbols.get(dom), 'achieved': achieved, 'peak': PEAK_BF16_TFLOPS, 'unit': 'TFLOP/s',
