@@ -82,7 +82,7 @@ template <int D, int MODE>
 __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     constexpr int KS = D / 16, DT = D / 32, PPR = D / 8;
     using L = Kv8Cfg<D, MODE>;
-    constexpr bool DK = L::DK, DV = L::DV, TWO = MODE == kKvBoth, SPLIT = MODE == kKvSplit;
+    constexpr bool DK = L::DK, TWO = MODE == kKvBoth, SPLIT = MODE == kKvSplit;
     static_assert(!TWO || D == 64, "both accumulators fit two waves per SIMD at D = 64 only");
     constexpr int PITCH = L::PITCH;
     __shared__ __attribute__((aligned(16))) char lds[L::LDS];
