@@ -249,15 +249,18 @@ def main():
     }
     if w2 <= 32:
         # the two-pass backward entry points, one pass (= one kernel) at a time
-        def one_pass(which, fn):
-            def run():
-                os.environ['SA2_BWD_PASS'] = which
-                try:
-                    return fn()
-                finally:
-                    del os.environ['SA2_BWD_PASS']
-            return run
-        launches['bwd_dq_dk2_pass'] = (3, one_pass('first', launches['bwd_dq_dkv2'][1]))
+        # the MFMA kernel of the dQ/dK2/dV2 entry point alone: the profiling build of the library
+        # launches only that kernel when SA2_BWD_PASS=first is set (the product library has no such switch)
+        plib = _native.load_profiling()
+
+        def dq_dk2_kernel_alone():
+            os.environ['SA2_BWD_PASS'] = 'first'
+            try:
+                return plib.sa2_bwd_dq_dkv2(prob, *five, arg(dout), lse.data_ptr(), delta.data_ptr(), saved, arg(dq),
+                                            arg(dk2), arg(dv2), ws.data_ptr(), ws_bytes, sh)
+            finally:
+                del os.environ['SA2_BWD_PASS']
+        launches['bwd_dq_dk2_pass'] = (3, dq_dk2_kernel_alone)
         # bwd_dkv1 is a single launch (one kernel produces dK1 and dV1)
     kernels = {}
     if args.only is not None:

@@ -13,6 +13,7 @@ import threading
 
 _CSRC = os.path.join(os.path.dirname(os.path.abspath(__file__)), 'csrc')
 LIB_PATH = os.path.join(_CSRC, 'libsa2.so')
+PROF_LIB_PATH = os.path.join(_CSRC, 'libsa2_prof.so')   # -DSA2_PROFILING build, for bench.py only
 
 SA2_OK = 0
 SA2_BF16 = 0
@@ -53,59 +54,73 @@ class Saved(ctypes.Structure):
 
 
 _lib = None
+_prof_lib = None
 _lock = threading.Lock()
 
 
 def build(verbose: bool = False) -> str:
     """Compile libsa2.so for gfx950 (always recompiles)."""
     out = None if verbose else subprocess.DEVNULL
-    subprocess.check_call(['make', '-B', '-C', _CSRC, 'libsa2.so'], stdout=out, stderr=out)
+    subprocess.check_call(['make', '-B', '-C', _CSRC, 'libsa2.so', 'libsa2_prof.so'], stdout=out, stderr=out)
     return LIB_PATH
+
+
+def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
+    P, T, F, V = ctypes.POINTER(Problem), ctypes.POINTER(TensorArg), ctypes.c_void_p, ctypes.c_void_p
+    S = ctypes.POINTER(Saved)
+    I64 = ctypes.c_int64
+    for name in ('sa2_saved_t_bytes', 'sa2_saved_m_bytes', 'sa2_bwd_workspace_bytes', 'sa2_qkv_norm_bwd_workspace_bytes'):
+        getattr(lib, name).restype = I64
+        getattr(lib, name).argtypes = [P]
+    lib.sa2_version.restype = ctypes.c_int
+    lib.sa2_version.argtypes = []
+    lib.sa2_last_error.restype = ctypes.c_char_p
+    lib.sa2_last_error.argtypes = []
+    lib.sa2_supported.restype = ctypes.c_int
+    lib.sa2_supported.argtypes = [ctypes.c_int32] * 4
+    lib.sa2_fwd.restype = ctypes.c_int
+    lib.sa2_fwd.argtypes = [P, T, T, T, T, T, T, T, F, S, V]
+    lib.sa2_bwd_delta.restype = ctypes.c_int
+    lib.sa2_bwd_delta.argtypes = [P, T, T, T, F, V]
+    lib.sa2_bwd_dq_dkv2.restype = ctypes.c_int
+    lib.sa2_bwd_dq_dkv2.argtypes = [P, T, T, T, T, T, T, F, F, S, T, T, T, V, I64, V]
+    lib.sa2_bwd_dkv1.restype = ctypes.c_int
+    lib.sa2_bwd_dkv1.argtypes = [P, T, T, T, T, T, T, F, F, T, T, V]
+    lib.sa2_bwd.restype = ctypes.c_int
+    lib.sa2_bwd.argtypes = [P, T, T, T, T, T, T, T, T, F, S, F, T, T, T, T, T, V, I64, V]
+    lib.sa2_qkv_norm_fwd.restype = ctypes.c_int
+    lib.sa2_qkv_norm_fwd.argtypes = [P, V, I64, V, V, V, V, V, ctypes.c_float, T, T, T, T, T, F, V]
+    lib.sa2_qkv_norm_bwd.restype = ctypes.c_int
+    lib.sa2_qkv_norm_bwd.argtypes = [P, V, I64, V, V, V, V, V, T, T, T, T, T, F, V, F, V, I64, V]
+    return lib
+
+
+def _missing(path: str) -> FileNotFoundError:
+    return FileNotFoundError(f'{path} is missing: build it with `make -C {_CSRC}` '
+                             '(or `python -c "import __graft_entry__ as g; g.build()"`)')
 
 
 def load() -> ctypes.CDLL:
     """Load libsa2.so and declare its prototypes.  Raises if it has not been built."""
     global _lib
     with _lock:
-        if _lib is not None:
-            return _lib
-        if not os.path.exists(LIB_PATH):
-            raise FileNotFoundError(
-                f'{LIB_PATH} is missing: build it with `make -C {_CSRC}` '
-                '(or `python -c "import __graft_entry__ as g; g.build()"`)')
-        lib = ctypes.CDLL(LIB_PATH)
-        P, T, F, V = ctypes.POINTER(Problem), ctypes.POINTER(TensorArg), ctypes.c_void_p, ctypes.c_void_p
-        S = ctypes.POINTER(Saved)
-        for name in ('sa2_saved_t_bytes', 'sa2_saved_m_bytes'):
-            getattr(lib, name).restype = ctypes.c_int64
-            getattr(lib, name).argtypes = [P]
-        lib.sa2_version.restype = ctypes.c_int
-        lib.sa2_version.argtypes = []
-        lib.sa2_last_error.restype = ctypes.c_char_p
-        lib.sa2_last_error.argtypes = []
-        lib.sa2_supported.restype = ctypes.c_int
-        lib.sa2_supported.argtypes = [ctypes.c_int32] * 4
-        lib.sa2_fwd.restype = ctypes.c_int
-        lib.sa2_fwd.argtypes = [P, T, T, T, T, T, T, T, F, S, V]
-        lib.sa2_bwd_delta.restype = ctypes.c_int
-        lib.sa2_bwd_delta.argtypes = [P, T, T, T, F, V]
-        lib.sa2_bwd_workspace_bytes.restype = ctypes.c_int64
-        lib.sa2_bwd_workspace_bytes.argtypes = [P]
-        lib.sa2_bwd_dq_dkv2.restype = ctypes.c_int
-        lib.sa2_bwd_dq_dkv2.argtypes = [P, T, T, T, T, T, T, F, F, S, T, T, T, V, ctypes.c_int64, V]
-        lib.sa2_bwd_dkv1.restype = ctypes.c_int
-        lib.sa2_bwd_dkv1.argtypes = [P, T, T, T, T, T, T, F, F, T, T, V]
-        lib.sa2_bwd.restype = ctypes.c_int
-        lib.sa2_bwd.argtypes = [P, T, T, T, T, T, T, T, T, F, S, F, T, T, T, T, T, V, ctypes.c_int64, V]
-        I64 = ctypes.c_int64
-        lib.sa2_qkv_norm_fwd.restype = ctypes.c_int
-        lib.sa2_qkv_norm_fwd.argtypes = [P, V, I64, V, V, V, V, V, ctypes.c_float, T, T, T, T, T, F, V]
-        lib.sa2_qkv_norm_bwd_workspace_bytes.restype = I64
-        lib.sa2_qkv_norm_bwd_workspace_bytes.argtypes = [P]
-        lib.sa2_qkv_norm_bwd.restype = ctypes.c_int
-        lib.sa2_qkv_norm_bwd.argtypes = [P, V, I64, V, V, V, V, V, T, T, T, T, T, F, V, F, V, I64, V]
-        _lib = lib
-        return lib
+        if _lib is None:
+            if not os.path.exists(LIB_PATH):
+                raise _missing(LIB_PATH)
+            _lib = _declare(ctypes.CDLL(LIB_PATH))
+        return _lib
+
+
+def load_profiling() -> ctypes.CDLL:
+    """The -DSA2_PROFILING build of the same sources: it honours SA2_BWD_PASS=first (launch only the
+    MFMA kernel of the dQ/dK2/dV2 entry point, results incomplete).  For kernel timing only."""
+    global _prof_lib
+    with _lock:
+        if _prof_lib is None:
+            if not os.path.exists(PROF_LIB_PATH):
+                raise _missing(PROF_LIB_PATH)
+            _prof_lib = _declare(ctypes.CDLL(PROF_LIB_PATH))
+        return _prof_lib
 
 
 def check(status: int) -> None:

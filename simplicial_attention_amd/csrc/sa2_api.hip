@@ -209,13 +209,14 @@ static int bwd_common(const sa2_problem *prob, const sa2_tensor *q, const sa2_te
     return SA2_OK;
 }
 
-// Profiling knob: SA2_BWD_PASS=first|second launches only one of the two passes of a
-// two-pass backward entry point (results are then incomplete); unset: both.
+// Profiling builds only (-DSA2_PROFILING, libsa2_prof.so): SA2_BWD_PASS=first launches only the
+// MFMA kernel of the dQ/dK2/dV2 entry point, so that it can be timed alone; the results of such a
+// call are incomplete.  The product library does not read the environment.
 static int bwd_pass_filter() {
+#ifdef SA2_PROFILING
     const char *v = std::getenv("SA2_BWD_PASS");
-    if (!v) return 0;
-    if (std::strcmp(v, "first") == 0) return 1;
-    if (std::strcmp(v, "second") == 0) return 2;
+    if (v && std::strcmp(v, "first") == 0) return 1;
+#endif
     return 0;
 }
 
@@ -250,10 +251,9 @@ int sa2_bwd_dq_dkv2(const sa2_problem *prob, const sa2_tensor *q, const sa2_tens
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
     const int grid = prob->batch * prob->heads * ((prob->seq_len + 31) / 32);
     const int w2max = qk2_w2max(prob->w2);
-    // offsets up to 32: two eight-wave passes (dq + dk2, then dv2); wider second windows (or
-    // SA2_BWD_QK2_IMPL=fused) take the fused four-wave kernel
-    const char *impl = std::getenv("SA2_BWD_QK2_IMPL");
-    const bool fused = w2max > 32 || (impl && std::strcmp(impl, "fused") == 0);
+    // offsets up to 32: two eight-wave passes (dq + dk2, then dv2); wider second windows take the
+    // fused four-wave kernel
+    const bool fused = w2max > 32;
     const int pass = bwd_pass_filter();
     // with the forward's saved per-offset T the dv2 pass (a recomputation of S and T) is
     // replaced by a kernel that streams T once
@@ -264,10 +264,10 @@ int sa2_bwd_dq_dkv2(const sa2_problem *prob, const sa2_tensor *q, const sa2_tens
         k.m_save = saved->m;
     }
     if (!fused && prob->dim_head == 128) {
-        if (pass != 2) hipLaunchKernelGGL((sa2::bwd_q8_kernel<128, true>), dim3(grid), dim3(512), 0, s, k, ws);
+        hipLaunchKernelGGL((sa2::bwd_q8_kernel<128, true>), dim3(grid), dim3(512), 0, s, k, ws);
         if (pass != 1 && !use_saved) hipLaunchKernelGGL((sa2::bwd_q8_kernel<128, false>), dim3(grid), dim3(512), 0, s, k, ws);
     } else if (!fused) {
-        if (pass != 2) hipLaunchKernelGGL((sa2::bwd_q8_kernel<64, true>), dim3(grid), dim3(512), 0, s, k, ws);
+        hipLaunchKernelGGL((sa2::bwd_q8_kernel<64, true>), dim3(grid), dim3(512), 0, s, k, ws);
         if (pass != 1 && !use_saved) hipLaunchKernelGGL((sa2::bwd_q8_kernel<64, false>), dim3(grid), dim3(512), 0, s, k, ws);
     } else if (prob->dim_head == 128 && w2max == 32)
         hipLaunchKernelGGL((sa2::bwd_qk2_kernel<128, 32>), dim3(grid), dim3(256), 0, s, k, ws);
@@ -308,33 +308,15 @@ int sa2_bwd_dkv1(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor 
     SA2_TRY(check_tensor(dv1, "dv1"));
     k.dk1 = dev(dk1);
     k.dv1 = dev(dv1);
-#ifdef SA2_TIMING
-    k.dq = dev(dk1);
-#endif
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
     int grid = prob->batch * prob->kv_heads * ((prob->seq_len + 127) / 128);
-    // offsets up to 32: eight-wave kernels, two passes (dk1, then dv1) at dim_head 128 and one
-    // kernel for both at dim_head 64; wider second windows (or SA2_BWD_KV1_IMPL=fused) take the
+    // offsets up to 32: one eight-wave kernel for both outputs; wider second windows take the
     // fused four-wave kernel
-    const char *impl = std::getenv("SA2_BWD_KV1_IMPL");
-    const bool fused = prob->w2 > 32 || (impl && std::strcmp(impl, "fused") == 0);
-    const int pass = bwd_pass_filter();
-    const char *split = std::getenv("SA2_BWD_KV1_SPLIT");           // profiling knob: dK1 and dV1 in two passes
-    if (!fused && prob->dim_head == 128) {
-        if (split && split[0] == '1') {
-            if (pass != 2) hipLaunchKernelGGL((sa2::bwd_kv8_kernel<128, sa2::kKvDk>), dim3(grid), dim3(512), 0, s, k);
-            if (pass != 1) hipLaunchKernelGGL((sa2::bwd_kv8_kernel<128, sa2::kKvDv>), dim3(grid), dim3(512), 0, s, k);
-        } else {
-            hipLaunchKernelGGL((sa2::bwd_kv8_kernel<128, sa2::kKvSplit>), dim3(grid), dim3(512), 0, s, k);
-        }
-    } else if (!fused) {
-        if (split && split[0] == '1') {
-            if (pass != 2) hipLaunchKernelGGL((sa2::bwd_kv8_kernel<64, sa2::kKvDk>), dim3(grid), dim3(512), 0, s, k);
-            if (pass != 1) hipLaunchKernelGGL((sa2::bwd_kv8_kernel<64, sa2::kKvDv>), dim3(grid), dim3(512), 0, s, k);
-        } else {
-            hipLaunchKernelGGL((sa2::bwd_kv8_kernel<64, sa2::kKvBoth>), dim3(grid), dim3(512), 0, s, k);
-        }
-    } else if (prob->dim_head == 128)
+    if (prob->w2 <= 32 && prob->dim_head == 128)
+        hipLaunchKernelGGL((sa2::bwd_kv8_kernel<128, sa2::kKvSplit>), dim3(grid), dim3(512), 0, s, k);
+    else if (prob->w2 <= 32)
+        hipLaunchKernelGGL((sa2::bwd_kv8_kernel<64, sa2::kKvBoth>), dim3(grid), dim3(512), 0, s, k);
+    else if (prob->dim_head == 128)
         hipLaunchKernelGGL(sa2::bwd_dkv1_kernel<128>, dim3(grid), dim3(256), 0, s, k);
     else
         hipLaunchKernelGGL(sa2::bwd_dkv1_kernel<64>, dim3(grid), dim3(256), 0, s, k);

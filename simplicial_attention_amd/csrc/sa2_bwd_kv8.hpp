@@ -125,20 +125,6 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     for (int dt = 0; dt < DT; ++dt) acc[dt] = zero16();
 #pragma unroll
     for (int dt = 0; dt < (TWO ? DT : 1); ++dt) acc2[dt] = zero16();
-#ifdef SA2_TIMING
-    long long t_acc[6] = {0, 0, 0, 0, 0, 0};
-    long long t_last = __builtin_amdgcn_s_memtime();
-#define TS(k)                                             \
-    {                                                     \
-        __builtin_amdgcn_sched_barrier(0);                \
-        const long long t_now = __builtin_amdgcn_s_memtime(); \
-        t_acc[k] += t_now - t_last;                       \
-        t_last = t_now;                                   \
-        __builtin_amdgcn_sched_barrier(0);                \
-    }
-#else
-#define TS(k)
-#endif
 
     const int it_begin = j0 / 32;
     const int last_i = (j0 + 127 + p.w1 - 1 < N - 1) ? j0 + 127 + p.w1 - 1 : N - 1;
@@ -472,7 +458,6 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
 
     for (int s = 0; s < npairs; ++s) {
         __syncthreads();
-        TS(0);
         if (s + 1 < npairs) {
             if (nb.m == 0) {
                 // the next pair opens a new query tile: its rows replace the staged ones
@@ -483,11 +468,9 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                 __syncthreads();
                 if constexpr (KEEP) unpack_own();
             }
-            TS(1);
             build(nb, (s + 1) & 1);
             next_pair(nb);
         }
-        TS(2);
         const char *buf = lds + (s & 1) * L::PAIR + pg * L::STEP;
         const int it = cur.it;
         next_pair(cur);
@@ -520,7 +503,6 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
             X[4 * a4 + 2] = X[4 * a4 + 2] * c2 - l4.z;
             X[4 * a4 + 3] = X[4 * a4 + 3] * c2 - l4.w;
         }
-        TS(3);
         const bool full = (jw + 31 <= 32 * it) && (jw + p.w1 > 32 * it + 31);
         if (!full) {
             const int base = 32 * it + 4 * hf - j;   // i - j for register 0
@@ -543,7 +525,6 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
             }
             pb[rr >> 3][(rr & 7) >> 1] = pack_bf16(p0, p1);
         }
-        TS(4);
 #pragma unroll
         for (int k2s = 0; k2s < 2; ++k2s)
 #pragma unroll
@@ -552,17 +533,8 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                 else acc[dt] = mfma32(tr_frag(buf + L::BS, BSwz{}, k2s, dt), pb[k2s], acc[dt]);
                 if constexpr (TWO) acc2[dt] = mfma32(tr_frag(buf + L::BS, BSwz{}, k2s, dt), pv[k2s], acc2[dt]);
             }
-        TS(5);
     }
 
-#ifdef SA2_TIMING
-    if (item == (int)gridDim.x / 2 + 3 && lane == 0) {
-        long long *dbg = reinterpret_cast<long long *>(p.dq.ptr) + (DK ? 0 : 64);
-        for (int k = 0; k < 6; ++k) dbg[wave * 8 + k] = t_acc[k];
-        dbg[wave * 8 + 6] = npairs;
-    }
-#endif
-#undef TS
     // ---- add the two groups of every slab and store
     __syncthreads();
     float *red = reinterpret_cast<float *>(lds) + (32 * slab + c) * L::RPITCH + 16 * hf;

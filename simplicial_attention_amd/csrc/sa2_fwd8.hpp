@@ -151,20 +151,6 @@ __global__ __launch_bounds__(512, (D == 64 && W2MAX == 32) ? 4 : 1) void fwd8_ke
         }
     }
 
-#ifdef SA2_TIMING
-    long long t_acc[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    long long t_last = __builtin_amdgcn_s_memtime();
-#define TS(k)                                                 \
-    {                                                         \
-        __builtin_amdgcn_sched_barrier(0);                    \
-        const long long t_now = __builtin_amdgcn_s_memtime(); \
-        t_acc[k] += t_now - t_last;                           \
-        t_last = t_now;                                       \
-        __builtin_amdgcn_sched_barrier(0);                    \
-    }
-#else
-#define TS(k)
-#endif
     f32x16 T[DT];
     u32x4 A[KS];
     float M = 0.f;             // private reference (log2 domain); meaningless while `seen` is -inf
@@ -196,7 +182,6 @@ __global__ __launch_bounds__(512, (D == 64 && W2MAX == 32) ? 4 : 1) void fwd8_ke
             for (int dt = 0; dt < DT; ++dt) T[dt] = zero16();
         }
 
-        TS(5);
         f32x16 X;
         float tmax = 0.f;
         u32x2 vf[DT][2][2];
@@ -278,7 +263,6 @@ __global__ __launch_bounds__(512, (D == 64 && W2MAX == 32) ? 4 : 1) void fwd8_ke
         };
         // barrier + refill of the ring behind the stage that becomes current
         auto sync_stage = [&]() {
-            TS(3);
             // stage u goes into its buffer (last read in step u-2) BEFORE the barrier that
             // publishes it: the writes fall into the time a wave would otherwise wait for the others
             if (u >= 1 && u_load - 1 >= u) {
@@ -286,10 +270,8 @@ __global__ __launch_bounds__(512, (D == 64 && W2MAX == 32) ? 4 : 1) void fwd8_ke
                 if (u_load < U) issue_loads();
             }
             __syncthreads();
-            TS(0);
             stage = lds + (u & 1) * C::STAGE;
             ++u;
-            TS(1);
         };
         // Runs chunks cc .. cc_end.  Returns true if it stopped inside chunk cc at sub-tile
         // `stop_x` because the logits in X left the safe range (nothing of that sub-tile
@@ -309,7 +291,6 @@ __global__ __launch_bounds__(512, (D == 64 && W2MAX == 32) ? 4 : 1) void fwd8_ke
                         return true;
                     }
                     seen = fmaxf(seen, tmax);
-                    TS(2);
                     finish_tile();
                 }
             }
@@ -346,7 +327,6 @@ __global__ __launch_bounds__(512, (D == 64 && W2MAX == 32) ? 4 : 1) void fwd8_ke
         }
 
         // ---- round end: agree on the common reference, add v2 * T into the shared rows
-        TS(3);
         {
             const bool fresh = seen == -INFINITY;
             if (hf == 0) xm[wave * 32 + c] = fresh ? -INFINITY : M + seen;
@@ -429,18 +409,7 @@ __global__ __launch_bounds__(512, (D == 64 && W2MAX == 32) ? 4 : 1) void fwd8_ke
                 __syncthreads();
             }
         }
-        TS(4);
     }
-#ifdef SA2_TIMING
-    const bool timed = item == (int)gridDim.x / 2 + 3 && p.o_lo.ptr;
-    if (timed && lane == 0) {
-        long long *dbg = reinterpret_cast<long long *>(p.o_lo.ptr + b * p.o_lo.sb + (int64_t)(i0 + wave) * p.o_lo.sn + h * p.o_lo.sh);
-        for (int k = 0; k < 6; ++k) dbg[k] = t_acc[k];
-        dbg[6] = U;
-        dbg[7] = R;
-    }
-#endif
-#undef TS
 
     // ---- output: O = acc_sh / L with L = sum_w l_w 2^(M_w - Mc)
     {
@@ -465,9 +434,6 @@ __global__ __launch_bounds__(512, (D == 64 && W2MAX == 32) ? 4 : 1) void fwd8_ke
         const float *src = acc_sh + row * C::APITCH + seg * SEG;
         char *orow = p.o.ptr + b * p.o.sb + (int64_t)ir * p.o.sn + h * p.o.sh + seg * SEG * 2;
         char *rrow = p.o_lo.ptr ? p.o_lo.ptr + b * p.o_lo.sb + (int64_t)ir * p.o_lo.sn + h * p.o_lo.sh + seg * SEG * 2 : nullptr;
-#ifdef SA2_TIMING
-        if (timed) rrow = nullptr;
-#endif
         float o[SEG];
 #pragma unroll
         for (int x = 0; x < SEG; x += 4) {

@@ -56,8 +56,15 @@ class SlidingTwoSimplicialAttention(Function):
         assert all(t.is_cuda for t in tensors), 'sliding-window 2-simplicial attention runs on the GPU only'
         if not causal:
             raise NotImplementedError('only causal=True is defined for the sliding windows')
-        if any(t.dtype != torch.bfloat16 for t in tensors):
-            raise TypeError('the MI355X kernels take bfloat16 activations; cast inputs with .bfloat16()')
+        in_dtype = q.dtype
+        if in_dtype not in (torch.bfloat16, torch.float16, torch.float32) or any(t.dtype != in_dtype for t in tensors):
+            raise TypeError('q, k1, k2, v1, v2 must share one dtype out of bfloat16, float16, float32')
+        # the kernels compute on bf16 operands with fp32 accumulation, as the reference's do for any input
+        # dtype (triton_two_simplicial_attention.py:110-112, 150-152); other dtypes are cast on the way in
+        # and results returned in the caller's dtype
+        if in_dtype is not torch.bfloat16:
+            tensors = tuple(t.to(torch.bfloat16) for t in tensors)
+            q, k1, k2, v1, v2 = tensors
         if q.dim() != 4:
             raise ValueError('expected (batch, seq, heads, dim_head) tensors')
         batch, seq_len, heads, dim = q.shape
@@ -96,13 +103,14 @@ class SlidingTwoSimplicialAttention(Function):
                                       _stream_handle(q.device)))
         ctx.save_for_backward(q, k1, k2, v1, v2, out, lse, residual, t_save, m_save)
         ctx.problem = (batch, seq_len, heads, kv_heads, dim, w1, w2, scale)
-        return out
+        ctx.in_dtype = in_dtype
+        return out if in_dtype is torch.bfloat16 else out.to(in_dtype)
 
     @staticmethod
     def backward(ctx, dout):
         q, k1, k2, v1, v2, out, lse, residual, t_save, m_save = ctx.saved_tensors
         batch, seq_len, heads, kv_heads, dim, w1, w2, scale = ctx.problem
-        dout = _unit_inner_stride(dout)
+        dout = _unit_inner_stride(dout if dout.dtype is torch.bfloat16 else dout.to(torch.bfloat16))
         lib = _native.load()
         delta = torch.empty_like(lse)
         dq = torch.empty_like(q)
@@ -119,6 +127,8 @@ class SlidingTwoSimplicialAttention(Function):
                                       delta.data_ptr(),
                                       arg(dq), arg(dk1), arg(dk2), arg(dv1), arg(dv2),
                                       workspace.data_ptr(), ws_bytes, _stream_handle(q.device)))
+        if ctx.in_dtype is not torch.bfloat16:
+            dq, dk1, dk2, dv1, dv2 = (t.to(ctx.in_dtype) for t in (dq, dk1, dk2, dv1, dv2))
         return dq, dk1, dk2, dv1, dv2, None, None, None, None
 
 

@@ -194,3 +194,31 @@ def test_bench_refuses_more_than_one_gpu():
     import subprocess, sys
     r = subprocess.run([sys.executable, os.path.join(ROOT, 'bench.py'), '--gpus', '2'], capture_output=True, text=True)
     assert r.returncode != 0 and 'one GPU' in r.stderr
+
+
+def test_product_library_reads_no_environment_switches(lib):
+    """Switches that skip launches (for kernel timing) exist in the profiling build only: the
+    library the package loads must not even contain their names."""
+    blob = open(_native.LIB_PATH, 'rb').read()
+    for name in (b'SA2_BWD_PASS', b'SA2_BWD_KV1_SPLIT', b'SA2_BWD_QK2_IMPL', b'SA2_BWD_KV1_IMPL'):
+        assert name not in blob, name
+    prof = open(_native.PROF_LIB_PATH, 'rb').read()
+    assert b'SA2_BWD_PASS' in prof
+
+
+def test_reference_import_paths_resolve_to_this_build():
+    """The import lines of the reference's README and tests work unchanged
+    (README.md:19, tests/test_triton.py:18, tests/test_attn.py:1-3 of the reference)."""
+    from simplicial_attention.triton_two_simplicial_attention import (
+        SlidingTwoSimplicialAttention, SlidingWindowTwoSimplicialMHA, sliding_two_simplicial_attn)
+    from simplicial_attention import naive_two_simplicial_attend, TwoSimplicialMHA, HigherOrderAttention
+    from simplicial_attention.simplicial_attention import naive_two_simplicial_attend as naive2
+    from simplicial_attention.simplicial_mha import HigherOrderAttention as HOA
+    from simplicial_attention.two_simplicial_transformer import TwoSimplicialTransformer
+    assert SlidingWindowTwoSimplicialMHA is S.SlidingWindowTwoSimplicialMHA
+    assert SlidingTwoSimplicialAttention is S.SlidingTwoSimplicialAttention
+    assert sliding_two_simplicial_attn is S.sliding_two_simplicial_attn
+    assert naive2 is naive_two_simplicial_attend is S.naive_two_simplicial_attend
+    assert HOA is HigherOrderAttention is S.HigherOrderAttention and TwoSimplicialMHA is S.TwoSimplicialMHA
+    attn = SlidingWindowTwoSimplicialMHA(dim=512, dim_head=64, heads=8)
+    assert isinstance(attn, HigherOrderAttention) and TwoSimplicialTransformer is not None

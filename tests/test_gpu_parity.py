@@ -131,18 +131,6 @@ def test_other_head_dimensions_and_dtypes(dtype, dqk, dv, n, w1, w2):
     U.check_all(out, grads, ref_out, ref_grads, unit_variance=True)
 
 
-@pytest.mark.parametrize('shape', [(2, 200, 4, 2, 64, 64, 32), (1, 300, 2, 2, 128, 96, 16)])
-def test_two_pass_key_value_backward(shape, monkeypatch):
-    """SA2_BWD_KV1_SPLIT=1: dK1 and dV1 from two passes (each recomputing S) instead of the
-    single kernel that produces both."""
-    monkeypatch.setenv('SA2_BWD_KV1_SPLIT', '1')
-    b, n, hq, hk, d, w1, w2 = shape
-    ins = U.make_inputs(b, n, hq, hk, d, seed=29, std=d ** -0.5)
-    ref_out, _, ref_grads = U.oracle_fwd_bwd(*ins, w1, w2)
-    out, grads = U.hip_fwd_bwd(*ins, w1, w2)
-    U.check_all(out, grads, ref_out, ref_grads)
-
-
 def test_backward_is_deterministic():
     ins = U.make_inputs(1, 384, 2, 1, 128, seed=11)
     first = U.hip_fwd_bwd(*ins, 128, 32)
