@@ -162,6 +162,27 @@ int sa2_bwd(const sa2_problem *prob,
             const sa2_tensor *dv1, const sa2_tensor *dv2,
             void *workspace, int64_t workspace_bytes, void *hip_stream);
 
+/* Whole backward for callers that cannot allocate (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): sa2_bwd without the delta_ws and workspace arguments.
+ * No counterpart in the reference.  The delta rows and the dK2/dV2 partial rows live in a
+ * device array of SA2_NOALLOC_SCRATCH_BYTES that is part of the library image (each GPU the
+ * library runs on holds one copy until the process ends); the call allocates and frees nothing.
+ * Problems that need more than that (sa2_bwd_noalloc_scratch_bytes() says how much) are refused
+ * with SA2_ERR_UNSUPPORTED: use sa2_bwd with caller-owned buffers.  All calls on one GPU share
+ * that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race; calls
+ * in stream order on one stream do not.  The array keeps the previous call's contents; nothing
+ * needs clearing because every element a kernel reads is written earlier in the same call.
+ * Results are bit-identical to sa2_bwd's. */
+#define SA2_NOALLOC_SCRATCH_BYTES (64ll << 20)
+int64_t sa2_bwd_noalloc_scratch_bytes(const sa2_problem *prob);   /* -1 if the problem is invalid */
+int sa2_bwd_noalloc(const sa2_problem *prob,
+                    const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
+                    const sa2_tensor *v1, const sa2_tensor *v2,
+                    const sa2_tensor *out, const sa2_tensor *out_residual, const sa2_tensor *dout,
+                    const float *lse, const sa2_saved *saved,
+                    const sa2_tensor *dq, const sa2_tensor *dk1, const sa2_tensor *dk2,
+                    const sa2_tensor *dv1, const sa2_tensor *dv2, void *hip_stream);
+
 /* ---- module pre-processing around the attention core (first of the "next" rows) ----
  *
  * Fused split + per-head RMSNorm of the qkv projection.  Replaces, for

@@ -27,6 +27,7 @@ STATUS_NAMES = {
 
 EXPORTS = ('sa2_version', 'sa2_last_error', 'sa2_supported', 'sa2_saved_t_bytes', 'sa2_saved_m_bytes', 'sa2_fwd',
            'sa2_bwd_delta', 'sa2_bwd_workspace_bytes', 'sa2_bwd_dq_dkv2', 'sa2_bwd_dkv1', 'sa2_bwd',
+           'sa2_bwd_noalloc_scratch_bytes', 'sa2_bwd_noalloc',
            'sa2_qkv_norm_fwd', 'sa2_qkv_norm_bwd_workspace_bytes', 'sa2_qkv_norm_bwd')
 
 
@@ -69,7 +70,8 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
     P, T, F, V = ctypes.POINTER(Problem), ctypes.POINTER(TensorArg), ctypes.c_void_p, ctypes.c_void_p
     S = ctypes.POINTER(Saved)
     I64 = ctypes.c_int64
-    for name in ('sa2_saved_t_bytes', 'sa2_saved_m_bytes', 'sa2_bwd_workspace_bytes', 'sa2_qkv_norm_bwd_workspace_bytes'):
+    for name in ('sa2_saved_t_bytes', 'sa2_saved_m_bytes', 'sa2_bwd_workspace_bytes', 'sa2_qkv_norm_bwd_workspace_bytes',
+                 'sa2_bwd_noalloc_scratch_bytes'):
         getattr(lib, name).restype = I64
         getattr(lib, name).argtypes = [P]
     lib.sa2_version.restype = ctypes.c_int
@@ -88,6 +90,8 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
     lib.sa2_bwd_dkv1.argtypes = [P, T, T, T, T, T, T, F, F, T, T, V]
     lib.sa2_bwd.restype = ctypes.c_int
     lib.sa2_bwd.argtypes = [P, T, T, T, T, T, T, T, T, F, S, F, T, T, T, T, T, V, I64, V]
+    lib.sa2_bwd_noalloc.restype = ctypes.c_int
+    lib.sa2_bwd_noalloc.argtypes = [P, T, T, T, T, T, T, T, T, F, S, T, T, T, T, T, V]
     lib.sa2_qkv_norm_fwd.restype = ctypes.c_int
     lib.sa2_qkv_norm_fwd.argtypes = [P, V, I64, V, V, V, V, V, ctypes.c_float, T, T, T, T, T, F, V]
     lib.sa2_qkv_norm_bwd.restype = ctypes.c_int

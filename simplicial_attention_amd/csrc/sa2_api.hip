@@ -8,6 +8,7 @@
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
+#include <mutex>
 
 #include "sa2_bwd.hpp"
 #include "sa2_bwd_kv8.hpp"
@@ -92,6 +93,34 @@ int after_launch(const char *what) {
         int rc_ = (expr);              \
         if (rc_ != SA2_OK) return rc_; \
     } while (0)
+
+// Scratch of sa2_bwd_noalloc: delta rows followed by the dK2/dV2 partial rows.  A file-scope device
+// array: every GPU the library runs on holds its own copy, at its own address, until the process
+// ends.  In host code the array's name is only a handle for hipGetSymbolAddress; kernels and
+// runtime calls get the address that call returns for the current device.
+constexpr int64_t kNoallocScratchBytes = SA2_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char g_noalloc_scratch[kNoallocScratchBytes];
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+unsigned char *g_scratch_ptr[kMaxDevices] = {};
+
+// device address of the scratch array on the current device (looked up once per device)
+int noalloc_scratch(unsigned char **out) {
+    int device = -1;
+    hipError_t e = hipGetDevice(&device);
+    if (e != hipSuccess) return fail(SA2_ERR_LAUNCH, "hipGetDevice failed: %s", hipGetErrorString(e));
+    if (device < 0 || device >= kMaxDevices) return fail(SA2_ERR_UNSUPPORTED, "device index %d is not supported (at most %d)", device, kMaxDevices);
+    std::lock_guard<std::mutex> guard(g_scratch_mutex);
+    if (!g_scratch_ptr[device]) {
+        void *ptr = nullptr;
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_noalloc_scratch));
+        if (e != hipSuccess || !ptr) return fail(SA2_ERR_LAUNCH, "hipGetSymbolAddress(scratch) failed: %s", hipGetErrorString(e));
+        g_scratch_ptr[device] = static_cast<unsigned char *>(ptr);
+    }
+    *out = g_scratch_ptr[device];
+    return SA2_OK;
+}
 
 }  // namespace
 
@@ -333,6 +362,34 @@ int sa2_bwd(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, 
                             workspace_bytes, hip_stream));
     SA2_TRY(sa2_bwd_dkv1(prob, q, k1, k2, v1, v2, dout, lse, delta_ws, dk1, dv1, hip_stream));
     return SA2_OK;
+}
+
+static int64_t align256(int64_t x) { return (x + 255) & ~int64_t(255); }
+
+int64_t sa2_bwd_noalloc_scratch_bytes(const sa2_problem *prob) {
+    const int64_t ws = sa2_bwd_workspace_bytes(prob);
+    if (ws < 0) return -1;
+    return align256((int64_t)prob->batch * prob->heads * prob->seq_len * 4) + ws;
+}
+
+int sa2_bwd_noalloc(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
+                    const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *out, const sa2_tensor *out_residual,
+                    const sa2_tensor *dout, const float *lse, const sa2_saved *saved, const sa2_tensor *dq,
+                    const sa2_tensor *dk1, const sa2_tensor *dk2, const sa2_tensor *dv1, const sa2_tensor *dv2,
+                    void *hip_stream) {
+    SA2_TRY(check_problem(prob));
+    const int64_t need = sa2_bwd_noalloc_scratch_bytes(prob);
+    if (need > kNoallocScratchBytes)
+        return fail(SA2_ERR_UNSUPPORTED, "this problem needs %lld bytes of scratch, the built-in buffer of sa2_bwd_noalloc holds %lld; "
+                    "use sa2_bwd with a caller-owned workspace", (long long)need, (long long)kNoallocScratchBytes);
+    unsigned char *scratch = nullptr;
+    SA2_TRY(noalloc_scratch(&scratch));
+    float *delta = reinterpret_cast<float *>(scratch);
+    unsigned char *ws = scratch + align256((int64_t)prob->batch * prob->heads * prob->seq_len * 4);
+    // every element of the scratch that a kernel reads was written by an earlier kernel of this same
+    // call (delta rows, partial rows), so nothing needs clearing between calls
+    return sa2_bwd(prob, q, k1, k2, v1, v2, out, out_residual, dout, lse, saved, delta, dq, dk1, dk2, dv1, dv2, ws,
+                   sa2_bwd_workspace_bytes(prob), hip_stream);
 }
 
 // ---- fused split + per-head RMSNorm of the qkv projection -------------------------------
