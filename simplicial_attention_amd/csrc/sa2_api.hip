@@ -17,6 +17,7 @@
 #include "sa2_common.hpp"
 #include "sa2_lds.hpp"
 #include "sa2_qkv_norm.hpp"
+#include "sa2_fwd.hpp"
 #include "sa2_fwd8.hpp"
 
 namespace {
@@ -178,15 +179,11 @@ int sa2_fwd(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, 
         k.m_save = saved->m;
     }
     const int grid = prob->batch * prob->heads * ((prob->seq_len + 31) / 32);
-    // the instance for second windows up to 32 stages fewer k2/v2 rows (at dim_head 64 two workgroups fit a CU)
-    const bool narrow = prob->w2 <= 32;
-    if (prob->dim_head == 128) {
-        if (narrow) hipLaunchKernelGGL((sa2::fwd8_kernel<128, 32>), dim3(grid), dim3(512), 0, s, k);
-        else hipLaunchKernelGGL((sa2::fwd8_kernel<128, 64>), dim3(grid), dim3(512), 0, s, k);
-    } else {
-        if (narrow) hipLaunchKernelGGL((sa2::fwd8_kernel<64, 32>), dim3(grid), dim3(512), 0, s, k);
-        else hipLaunchKernelGGL((sa2::fwd8_kernel<64, 64>), dim3(grid), dim3(512), 0, s, k);
-    }
+    // dim_head 64 with a second window of up to 32: the instance that fits four waves per SIMD
+    // (two workgroups per CU); everything else: the general kernel (any second window)
+    if (prob->dim_head == 128) hipLaunchKernelGGL(sa2::fwd_kernel<128>, dim3(grid), dim3(512), 0, s, k);
+    else if (prob->w2 <= 32) hipLaunchKernelGGL((sa2::fwd8_kernel<64, 32>), dim3(grid), dim3(512), 0, s, k);
+    else hipLaunchKernelGGL(sa2::fwd_kernel<64>, dim3(grid), dim3(512), 0, s, k);
     return after_launch("forward");
 }
 

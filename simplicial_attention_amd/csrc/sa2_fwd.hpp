@@ -1,0 +1,542 @@
+// Forward kernel (eight waves, two per SIMD).
+//
+// One workgroup owns 32 query rows of one (batch, head).  In round r wave w handles the
+// offset dlt = i - k = 8r + w (any second window: ceil(w2 / 8) rounds); all eight waves walk
+// the same 32-row K1/V1 tiles, which stream through a three-buffer LDS ring, one tile and
+// one barrier per step.  Per (offset, tile):
+//     S^T = K1 A^T          A = q_i * k2_{i-dlt} * scale * log2(e)   (bf16, built once per offset)
+//     P^T = exp2(S^T - M_i)                 (the MFMA chain starts from -M_i: no VALU subtraction)
+//     T^T += V1^T P^T       (V1 fragments through ds_read_b64_tr_b16)
+// Measured on MI355X: a wave hides about four plain VALU instructions behind each of its own
+// 32x32x16 MFMAs and none beyond that, and a second wave on the SIMD fills the MFMA pipe while
+// the first one runs its exponentials - provided that phase is shorter than an MFMA phase.
+// So the per-tile VALU work is kept to the exponentials, the bf16 packing and the row sums:
+//   - the softmax reference M of a row is fixed by the first tile of the wave's first offset
+//     (the diagonal tile, which every valid row attends) and moves only when a row sum says
+//     that weights grew beyond 2^90 (a branch that is almost never taken);
+//   - masks are applied on the diagonal tile and on the (at most two) tiles that the window's
+//     lower edge crosses; the tiles in between run without mask code;
+//   - the V1 fragments of a tile are requested when its logit chain has been issued and arrive
+//     behind the exponentials; the K1 fragments of the next tile are requested in front of the
+//     value chain and arrive behind it and the barrier.
+// The output accumulator is shared: an fp32 [32][D] LDS buffer relative to a common reference
+// Mc.  At the end of a round the waves publish their references, agree on Mc = max, and add
+// v2_{i-dlt} * T * 2^(M - Mc) in eight barrier-separated phases; in phase ph wave w owns the
+// d-slice (w + ph) mod 8, so concurrent waves never touch the same element and every element
+// sees its additions in a fixed order (bitwise reproducible, no atomics).
+// The k2/v2 rows live in a 64-row circular LDS buffer (row k in slot (k - i0) mod 64): a round
+// needs 39 of them and the 8 rows that the next round adds are fetched while the round's results
+// are added to the shared accumulator.
+#pragma once
+
+#include <type_traits>
+
+#include "sa2_common.hpp"
+#include "sa2_lds.hpp"
+
+namespace sa2 {
+
+template <int D>
+struct FwdCfg {
+    static constexpr int KS = D / 16;
+    static constexpr int DT = D / 32;
+    static constexpr int PITCH = tile_pitch<D>();
+    static constexpr int TILE = 32 * PITCH;           // K1 tile, read row-major
+    static constexpr int VPITCH = tr_pitch<D>();
+    static constexpr int VTILE = 32 * VPITCH;         // V1 tile, read through transposed reads only
+    static constexpr int BUF = TILE + VTILE;          // one ring buffer: a K1 tile and a V1 tile
+    static constexpr int NBUF = 3;
+    static constexpr int RING = NBUF * BUF;
+    static constexpr int APITCH = D + 4;              // floats per row of the shared accumulator
+    static constexpr int ACC = 32 * APITCH * 4;
+    static constexpr int EXCH = 8 * 32 * 4;           // one float per (wave, row)
+    static constexpr int QS = RING + ACC + 2 * EXCH;  // q rows of the tile      [32][PITCH]
+    static constexpr int KSLOTS = 64;                 // circular k2 / v2 rows
+    static constexpr int K2S = QS + TILE;
+    static constexpr int V2S = K2S + KSLOTS * PITCH;
+    static constexpr int MASKS = V2S + KSLOTS * PITCH; // additive masks (0 / -inf) of the diagonal tile and of up to two lower-edge tiles
+    static constexpr int MASK = 16 * 64 * 4;          // one table: [4 quarters][64 lanes][4 floats]
+    static constexpr int LDS = MASKS + 3 * MASK;
+    static constexpr int PPR = D / 8;                 // 16-byte pieces per row
+    static constexpr int PIECES = 32 * PPR;           // ... per tile
+};
+
+template <int D>
+__global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
+    using C = FwdCfg<D>;
+    constexpr int KS = C::KS, DT = C::DT, PPR = C::PPR, PITCH = C::PITCH;
+    constexpr float kBig = 1.2379400392853803e27f;    // 2^90: row sums beyond it move the reference
+    __shared__ __attribute__((aligned(16))) char lds[C::LDS];
+
+    const int N = p.N;
+    const int ntile = (N + 31) / 32;
+    const int item = xcd_contiguous(blockIdx.x, gridDim.x);
+    const int tile = ntile - 1 - item % ntile;
+    const int bh = item / ntile;
+    const int h = bh % p.H, b = bh / p.H;
+    const int hk = h / p.G;
+
+    const int tid = threadIdx.x;
+    const int wave = wave_index(), lane = tid & 63;
+    const int c = lane & 31, hf = lane >> 5;
+    const int i0 = tile * 32;
+    const int i = i0 + c;
+    const bool row_ok = i < N;
+
+    const char *k1g = p.k1.ptr + b * p.k1.sb + hk * p.k1.sh;
+    const char *v1g = p.v1.ptr + b * p.v1.sb + hk * p.v1.sh;
+    const char *k2g = p.k2.ptr + b * p.k2.sb + hk * p.k2.sh;
+    const char *v2g = p.v2.ptr + b * p.v2.sb + hk * p.v2.sh;
+
+    // tiles of the first window; sequence of a round: the diagonal tile first, then t_lo .. t_hi - 1
+    const int t_lo = (i0 - p.w1 + 1 > 0 ? i0 - p.w1 + 1 : 0) / 32;
+    const int t_hi = i0 / 32;
+    const int NT = t_hi - t_lo + 1;
+    int mid_lo = (i0 + 31 - p.w1 >= 0) ? (i0 + 31 - p.w1) / 32 + 1 : t_lo;   // first tile below the diagonal that no row masks
+    mid_lo = mid_lo > t_hi ? t_hi : mid_lo;
+    const int n_masked = 1 + (mid_lo - t_lo);         // leading steps of a round that need a mask (at most 3)
+    const int nd = p.w2 < i0 + 32 ? p.w2 : i0 + 32;   // offsets that meet at least one valid k
+    const int R = (nd + 7) / 8;
+    const int U = R * NT;
+    auto tile_of = [&](int n) { return n == 0 ? t_hi : t_lo + n - 1; };
+
+    // ---- ring staging: the first PIECES threads move one 16-byte piece of K1 and of V1 per tile
+    const bool stager = tid < C::PIECES;
+    const int st_row = tid / PPR, st_col = (tid % PPR) * 16;
+    const int st_off = st_row * PITCH + st_col;
+    const int st_off_v = C::TILE + st_row * C::VPITCH + st_col;
+    u32x4 st_k = {0u, 0u, 0u, 0u}, st_v = {0u, 0u, 0u, 0u};
+    int n_load = 0, u_load = 0;                       // sequence index (within the round) / running count of the next load
+    // address = tile base (uniform, on the scalar unit) + this thread's row and column (32 bits); only
+    // the diagonal tile can reach past the last row, so only it needs a clamped row
+    const int st_row_diag = i0 + st_row < N ? st_row : N - 1 - i0;
+    const uint32_t so_k = (uint32_t)(st_row * (int)p.k1.sn + st_col), so_v = (uint32_t)(st_row * (int)p.v1.sn + st_col);
+    const uint32_t so_k_diag = (uint32_t)(st_row_diag * (int)p.k1.sn + st_col), so_v_diag = (uint32_t)(st_row_diag * (int)p.v1.sn + st_col);
+    auto issue_loads = [&]() {
+        const int t = tile_of(n_load);
+        const char *kb = k1g + (int64_t)(32 * t) * p.k1.sn;
+        const char *vb = v1g + (int64_t)(32 * t) * p.v1.sn;
+        if (stager) {
+            st_k = ld_global16(kb + (n_load == 0 ? so_k_diag : so_k));
+            st_v = ld_global16(vb + (n_load == 0 ? so_v_diag : so_v));
+        }
+        ++u_load;
+        n_load = (n_load == NT - 1) ? 0 : n_load + 1;
+    };
+    auto write_stage = [&](int buf_off) {
+        if (stager) {
+            *reinterpret_cast<u32x4 *>(lds + buf_off + st_off) = st_k;
+            *reinterpret_cast<u32x4 *>(lds + buf_off + st_off_v) = st_v;
+        }
+    };
+    const int k_lane = c * PITCH + 16 * hf;          // K1 fragment: row c, pieces 2*kk + hf
+    const int v_lane = C::TILE + tr_lane_off<D, C::VPITCH>(lane);
+
+    // ---- shared output accumulator and exchange areas
+    float *acc_sh = reinterpret_cast<float *>(lds + C::RING);              // [32][APITCH]
+    float *xm = reinterpret_cast<float *>(lds + C::RING + C::ACC);         // [8][32] references
+    float *xl = xm + 8 * 32;                                               // [8][32] row sums
+    for (int x = tid; x < 32 * C::APITCH / 4; x += 512) reinterpret_cast<float4 *>(acc_sh)[x] = make_float4(0.f, 0.f, 0.f, 0.f);
+    float Mc = -INFINITY;      // common reference of acc_sh (same value in every wave)
+
+    // ---- the q rows of the tile and the k2/v2 rows of the first round, staged before the loop
+    {
+        const char *qg = p.q.ptr + b * p.q.sb + h * p.q.sh;
+        for (int x = tid; x < 32 * PPR; x += 512) {
+            const int row = x / PPR, col = (x % PPR) * 16;
+            int ii = i0 + row;
+            ii = ii < N ? ii : N - 1;
+            *reinterpret_cast<u32x4 *>(lds + C::QS + row * PITCH + col) = ld_global16(qg + (int64_t)ii * p.q.sn + col);
+        }
+        for (int x = tid; x < 39 * PPR; x += 512) {
+            const int row = x / PPR, col = (x % PPR) * 16;
+            int kk2 = i0 - 7 + row;
+            kk2 = kk2 < 0 ? 0 : (kk2 < N ? kk2 : N - 1);
+            const int slot = (row - 7) & 63;
+            *reinterpret_cast<u32x4 *>(lds + C::K2S + slot * PITCH + col) = ld_global16(k2g + (int64_t)kk2 * p.k2.sn + col);
+            *reinterpret_cast<u32x4 *>(lds + C::V2S + slot * PITCH + col) = ld_global16(v2g + (int64_t)kk2 * p.v2.sn + col);
+        }
+    }
+    // additive masks: table 0 for the diagonal tile, tables 1, 2 for the tiles the lower window edge
+    // crosses.  Entry (lane, rr) is 0 if query row i0 + c attends key row 32 t + 4 hf + e(rr), else -inf
+    for (int x = tid; x < 3 * 256; x += 512) {
+        const int tab = x >> 8, qq = (x >> 6) & 3, ln = x & 63;
+        const int t = tab == 0 ? t_hi : t_lo + tab - 1;
+        const int rel = (ln & 31) + 32 * (t_hi - t) - 4 * (ln >> 5);
+        float4 m4;
+        float *mp = &m4.x;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) mp[e] = ((unsigned)(rel - (8 * qq + e)) < (unsigned)p.w1) ? 0.f : -INFINITY;
+        *reinterpret_cast<float4 *>(lds + C::MASKS + tab * C::MASK + qq * 1024 + ln * 16) = m4;
+    }
+    // the 8 rows that round r + 1 adds (k - i0 = -8r - 15 .. -8r - 8), one 16-byte piece per thread
+    const bool row_stager = tid < 2 * 8 * PPR;
+    const int rs_sel = tid / (8 * PPR), rs_row = (tid / PPR) % 8, rs_col = (tid % PPR) * 16;
+    u32x4 st_r = {0u, 0u, 0u, 0u};
+    auto issue_rows = [&](int r) {
+        if (row_stager) {
+            int kk2 = i0 - 8 * r - 15 + rs_row;
+            kk2 = kk2 < 0 ? 0 : (kk2 < N ? kk2 : N - 1);
+            st_r = ld_global16((rs_sel ? v2g + (int64_t)kk2 * p.v2.sn : k2g + (int64_t)kk2 * p.k2.sn) + rs_col);
+        }
+    };
+    auto write_rows = [&](int r) {
+        if (row_stager) {
+            const int slot = (-8 * r - 15 + rs_row) & 63;
+            *reinterpret_cast<u32x4 *>(lds + (rs_sel ? C::V2S : C::K2S) + slot * PITCH + rs_col) = st_r;
+        }
+    };
+
+    f32x16 T[DT];
+    u32x4 A[KS];
+    u32x4 kf[KS];              // K1 fragments of the step about to run (requested at the end of the step before, or at the round's start)
+    u32x2 vf[DT][2][2];        // V1 fragments of the running step (requested when its logit chain has been issued)
+    float M = 0.f;             // softmax reference of the row (log2 domain); meaningless while `fresh`
+    bool fresh = true;         // the row has not met an attended entry yet
+    float l = 0.f;             // this lane's part of the row sum, relative to M
+
+    // ring protocol: step u lives in buffer u % 3; it is written at the end of step u - 2 from
+    // registers loaded at the end of step u - 3 and read (as fragments) from step u - 1 on
+    int b_cur = 0, b_nxt = C::BUF, b_nn = 2 * C::BUF;
+    issue_loads();
+    write_stage(0);
+    if (U > 1) {
+        issue_loads();
+        write_stage(C::BUF);
+    }
+    if (U > 2) issue_loads();
+    int u = 0;
+
+    // end of a step: the tile two steps ahead goes to its buffer, the next global loads start
+    auto stage_ahead = [&]() {
+        if (u + 2 < U) {
+            write_stage(b_nn);
+            if (u_load < U) issue_loads();
+        }
+        const int t = b_cur;
+        b_cur = b_nxt;
+        b_nxt = b_nn;
+        b_nn = t;
+        ++u;
+    };
+
+    __syncthreads();           // staged rows, the zeroed accumulator and the first two tiles are visible
+
+    for (int r = 0; r < R; ++r) {
+        const int dlt = 8 * r + wave;
+        const int kr = i - dlt;
+        const bool col_ok = row_ok && kr >= 0 && dlt < p.w2;
+        const bool wave_on = wave_any(col_ok);
+        const int slot = (c - dlt) & 63;              // slot of row k = i - dlt in the circular k2/v2 rows
+        {
+            const char *k2row = lds + C::K2S + slot * PITCH + 16 * hf;
+            const char *qr = lds + C::QS + c * PITCH + 16 * hf;
+            const float c2 = p.scale_log2e;
+#pragma unroll
+            for (int kk = 0; kk < KS; ++kk) {
+                const u32x4 fq = ld_lds16(qr + 32 * kk), fk = ld_lds16(k2row + 32 * kk);
+#pragma unroll
+                for (int w = 0; w < 4; ++w)
+                    A[kk][w] = pack_bf16(bf16_lo(fq[w]) * bf16_lo(fk[w]) * c2, bf16_hi(fq[w]) * bf16_hi(fk[w]) * c2);
+            }
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) T[dt] = zero16();
+        }
+
+        // exponentials and row sums of the tile whose referenced logits are in X
+        auto exponentials = [&](const f32x16 &X, u32x4 (&pb)[2]) {
+            // (the row sum takes the unrounded weights: v_dot2c_f32_bf16 on the packed pairs would be exact
+            // for what the MFMA consumes, but dot instructions share the MFMA pipe and stall the other
+            // wave's chains; the two sums differ by the mean of bf16 rounding errors, far below bf16 eps)
+            float ls = 0.f;
+#pragma unroll
+            for (int rr = 0; rr < 16; rr += 2) {
+                const float e0 = fast_exp2(X[rr]), e1 = fast_exp2(X[rr + 1]);
+                ls += e0 + e1;
+                pb[rr >> 3][(rr & 7) >> 1] = pack_bf16(e0, e1);
+            }
+            l += ls;
+        };
+        // fragment reads of a step: the V1 fragments of the tile behind its logit chain, the K1 fragments of
+        // the next tile in front of the value chain (they arrive behind it and the barrier)
+        auto load_vf = [&]() {
+            const char *vbase = lds + b_cur + v_lane;
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int k2s = 0; k2s < 2; ++k2s) {
+                    vf[dt][k2s][0] = lds_read_tr<D, C::VPITCH>(vbase, 16 * k2s, 32 * dt);
+                    vf[dt][k2s][1] = lds_read_tr<D, C::VPITCH>(vbase, 16 * k2s + 8, 32 * dt);
+                }
+        };
+        auto load_kf = [&](int buf_off) {
+            const char *kbase = lds + buf_off + k_lane;
+#pragma unroll
+            for (int kk = 0; kk < KS; ++kk) kf[kk] = ld_lds16(kbase + 32 * kk);
+        };
+        auto value_products = [&](const u32x4 (&pb)[2], bool next_kf) {
+            if (next_kf) load_kf(b_nxt);
+#pragma unroll
+            for (int k2s = 0; k2s < 2; ++k2s)
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    u32x4 v = {vf[dt][k2s][0][0], vf[dt][k2s][0][1], vf[dt][k2s][1][0], vf[dt][k2s][1][1]};
+                    T[dt] = mfma32(v, pb[k2s], T[dt]);
+                }
+        };
+        // S^T = K1 A^T on top of X
+        auto logit_chain = [&](f32x16 &X) {
+#pragma unroll
+            for (int kk = 0; kk < KS; ++kk) X = mfma32(kf[kk], A[kk], X);
+            load_vf();
+        };
+        // moves the reference of this lane's row up by `shift` (log2 units): what T and l hold is rescaled
+        // (alpha = 2^-shift, or 1 for a row that holds nothing yet)
+        auto shift_reference = [&](float shift, float alpha, f32x16 &X) {
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                for (int rr = 0; rr < 16; ++rr) T[dt][rr] *= alpha;
+#pragma unroll
+            for (int rr = 0; rr < 16; ++rr) X[rr] -= shift;
+            l *= alpha;
+            M += shift;
+        };
+        auto row_max = [&](const f32x16 &X) {
+            float tmax = X[0];
+#pragma unroll
+            for (int rr = 1; rr < 16; ++rr) tmax = fmaxf(tmax, X[rr]);
+            auto sw = __builtin_amdgcn_permlane32_swap(as_u32(tmax), as_u32(tmax), false, false);
+            return fmaxf(as_f32(sw[0]), as_f32(sw[1]));
+        };
+
+        if (wave_on) load_kf(b_cur);    // the round's first tile (its buffer was published at least one barrier ago)
+        if (!wave_on) {
+            // no valid (row, offset) in this wave: it only keeps the ring going
+            // (a wave that is off stays off: later rounds only have larger offsets, so its fragment
+            // registers need not follow the ring)
+            for (int n = 0; n < NT; ++n) {
+                __syncthreads();
+                stage_ahead();
+            }
+        } else {
+            int n = 0;
+            if (r == 0) {
+                // ---- the wave's very first step, the diagonal tile of its first offset: every valid row
+                // attends an entry of it, so this is where the rows get their softmax reference M
+                __syncthreads();
+                f32x16 X = zero16();
+                logit_chain(X);
+                {
+                    // row j = 32 t + 4 hf + e (e = 8 (rr / 4) + rr % 4) is attended iff 0 <= i - j < w1;
+                    // lanes without a valid k2 row get a distance no e can bring into range
+                    const int rel = col_ok ? c - 4 * hf : -(1 << 30);
+#pragma unroll
+                    for (int rr = 0; rr < 16; ++rr) {
+                        const bool ok = (unsigned)(rel - (8 * (rr >> 2) + (rr & 3))) < (unsigned)p.w1;
+                        X[rr] = ok ? X[rr] : -INFINITY;
+                    }
+                }
+                const float tmax = row_max(X);
+                if (tmax > -INFINITY) {
+                    M = tmax;
+                    fresh = false;
+#pragma unroll
+                    for (int rr = 0; rr < 16; ++rr) X[rr] -= tmax;
+                }
+                u32x4 pb[2];
+                exponentials(X, pb);
+                value_products(pb, 1 < NT);
+                stage_ahead();
+                n = 1;
+            }
+            // ---- all other steps.  The logit chain starts from -M (from -inf in lanes without a valid
+            // (row, offset)), plus an additive 0 / -inf mask from an LDS table on the diagonal tile and on the
+            // tiles that the window's lower edge crosses, so its result is the exponent and no mask or
+            // subtraction code follows it.  A row's reference moves only if its row sum says that weights
+            // outgrew the safe range.
+            // The two waves of a SIMD advance in step (their dependent MFMA chains interleave one
+            // instruction at a time), so with the barrier at the same place both would run their
+            // exponentials at the same time and leave the MFMA pipe idle.  The second wave of each SIMD
+            // (waves 4-7) therefore takes the step's barrier after its logit chain instead of before it:
+            // behind every barrier the first group starts a logit chain while the second group starts its
+            // exponentials.  Reading tile n before the step's barrier is safe: the barrier before published it.
+            const bool late = wave >= 4;
+            float nm = col_ok ? -M : -INFINITY;
+            u32x4 pb[2];
+            for (; n < NT; ++n) {
+                if (!late) __syncthreads();
+                f32x16 X;
+                if (n < n_masked) {
+                    const char *mk = lds + C::MASKS + n * C::MASK + lane * 16;
+#pragma unroll
+                    for (int qq = 0; qq < 4; ++qq) {
+                        const float4 m4 = *reinterpret_cast<const float4 *>(mk + qq * 1024);
+                        X[4 * qq] = m4.x + nm;
+                        X[4 * qq + 1] = m4.y + nm;
+                        X[4 * qq + 2] = m4.z + nm;
+                        X[4 * qq + 3] = m4.w + nm;
+                    }
+                } else {
+#pragma unroll
+                    for (int rr = 0; rr < 16; ++rr) X[rr] = nm;
+                }
+                logit_chain(X);
+                if (late) __syncthreads();
+                const float l_before = l;
+                exponentials(X, pb);
+                if (wave_any(!(l < kBig))) {
+                    // rare: some row's weights outgrew the safe range; move its reference and redo the tile's weights
+                    const float tmax = row_max(X);
+                    auto sw = __builtin_amdgcn_permlane32_swap(as_u32(l), as_u32(l), false, false);
+                    const float l_row = fmaxf(as_f32(sw[0]), as_f32(sw[1]));
+                    const bool over = !(l_row < kBig);
+                    l = l_before;
+                    const float lb = fmaxf(l_before, 1.f);
+                    auto sw2 = __builtin_amdgcn_permlane32_swap(as_u32(lb), as_u32(lb), false, false);
+                    const float e_old = (float)(__builtin_amdgcn_frexp_expf(fmaxf(as_f32(sw2[0]), as_f32(sw2[1]))) - 32);
+                    const float shift = over ? fmaxf(fmaxf(tmax, e_old), 0.f) : 0.f;
+                    shift_reference(shift, fast_exp2(-shift), X);
+                    nm = col_ok ? -M : -INFINITY;
+                    exponentials(X, pb);
+                }
+                value_products(pb, n + 1 < NT);
+                stage_ahead();
+            }
+        }
+
+        // ---- round end: agree on the common reference, add v2 * T into the shared rows
+        {
+            if (r + 1 < R) issue_rows(r);      // the rows that the next round adds arrive behind the phases below
+            if (hf == 0) xm[wave * 32 + c] = fresh ? -INFINITY : M;
+            __syncthreads();
+            float Mn = Mc;
+#pragma unroll
+            for (int w = 0; w < 8; ++w) Mn = fmaxf(Mn, xm[w * 32 + c]);
+            const float fo = (Mc == -INFINITY) ? 0.f : fast_exp2(Mc - Mn);   // rescale of the old content
+            const float g = (fresh || !wave_on) ? 0.f : fast_exp2(M - Mn);   // weight of this wave's T
+            // by-product for the backward: this offset's T and its reference
+            if (p.t_save && row_ok && dlt < p.w2) {
+                const int64_t srow_g = (((int64_t)b * p.H + h) * p.w2 + dlt) * N + i;
+                char *trow = p.t_save + srow_g * (D * 2) + 16 * hf * 2;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt) {
+                    u32x4 lo4, hi4;
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) {
+                        lo4[w] = pack_bf16(T[dt][2 * w], T[dt][2 * w + 1]);
+                        hi4[w] = pack_bf16(T[dt][8 + 2 * w], T[dt][8 + 2 * w + 1]);
+                    }
+                    st_global16(trow + dt * 64, lo4);
+                    st_global16(trow + dt * 64 + 16, hi4);
+                }
+                if (hf == 0) p.m_save[srow_g] = fresh ? 0.f : M;
+            }
+            Mc = Mn;
+            const char *v2row = lds + C::V2S + slot * PITCH + 16 * hf * 2;
+            float *arow = acc_sh + c * C::APITCH + 16 * hf;
+            auto add_slice = [&](auto slice_tag, bool first) {
+                constexpr int S = decltype(slice_tag)::value;     // slice: dt = S / 2, registers 8*(S%2) .. +7
+                constexpr int dt = S >> 1, r0 = 8 * (S & 1);
+                const u32x4 xv = ld_lds16(v2row + dt * 64 + r0 * 2);
+                float *dst = arow + 32 * dt + r0;
+                float4 a0 = *reinterpret_cast<float4 *>(dst), a1 = *reinterpret_cast<float4 *>(dst + 4);
+                if (first) {
+                    a0.x *= fo; a0.y *= fo; a0.z *= fo; a0.w *= fo;
+                    a1.x *= fo; a1.y *= fo; a1.z *= fo; a1.w *= fo;
+                }
+                a0.x += bf16_lo(xv[0]) * T[dt][r0] * g;
+                a0.y += bf16_hi(xv[0]) * T[dt][r0 + 1] * g;
+                a0.z += bf16_lo(xv[1]) * T[dt][r0 + 2] * g;
+                a0.w += bf16_hi(xv[1]) * T[dt][r0 + 3] * g;
+                a1.x += bf16_lo(xv[2]) * T[dt][r0 + 4] * g;
+                a1.y += bf16_hi(xv[2]) * T[dt][r0 + 5] * g;
+                a1.z += bf16_lo(xv[3]) * T[dt][r0 + 6] * g;
+                a1.w += bf16_hi(xv[3]) * T[dt][r0 + 7] * g;
+                *reinterpret_cast<float4 *>(dst) = a0;
+                *reinterpret_cast<float4 *>(dst + 4) = a1;
+            };
+            for (int ph = 0; ph < 8; ++ph) {
+                if constexpr (DT == 4) {
+                    switch ((wave + ph) & 7) {
+                        case 0: add_slice(std::integral_constant<int, 0>{}, ph == 0); break;
+                        case 1: add_slice(std::integral_constant<int, 1>{}, ph == 0); break;
+                        case 2: add_slice(std::integral_constant<int, 2>{}, ph == 0); break;
+                        case 3: add_slice(std::integral_constant<int, 3>{}, ph == 0); break;
+                        case 4: add_slice(std::integral_constant<int, 4>{}, ph == 0); break;
+                        case 5: add_slice(std::integral_constant<int, 5>{}, ph == 0); break;
+                        case 6: add_slice(std::integral_constant<int, 6>{}, ph == 0); break;
+                        default: add_slice(std::integral_constant<int, 7>{}, ph == 0); break;
+                    }
+                } else {
+                    // D = 64: four slices; waves 0-3 use phases 0-3, waves 4-7 phases 4-7
+                    if ((ph >> 2) == (wave >> 2)) {
+                        switch ((wave + ph) & 3) {
+                            case 0: add_slice(std::integral_constant<int, 0>{}, ph == 0); break;
+                            case 1: add_slice(std::integral_constant<int, 1>{}, ph == 0); break;
+                            case 2: add_slice(std::integral_constant<int, 2>{}, ph == 0); break;
+                            default: add_slice(std::integral_constant<int, 3>{}, ph == 0); break;
+                        }
+                    }
+                }
+                if (ph == 7 && r + 1 < R) write_rows(r);    // (their slots are not in use in this round)
+                __syncthreads();
+            }
+        }
+    }
+
+    // ---- output: O = acc_sh / L with L = sum_w l_w 2^(M_w - Mc)
+    {
+        auto sw = __builtin_amdgcn_permlane32_swap(as_u32(l), as_u32(l), false, false);
+        const float l_tot = as_f32(sw[0]) + as_f32(sw[1]);
+        if (hf == 0) {
+            xl[wave * 32 + c] = fresh ? 0.f : l_tot * fast_exp2(M - Mc);
+            if (wave == 0) xm[c] = Mc;
+        }
+    }
+    __syncthreads();
+    {
+        constexpr int SEG = D / 16;             // d values per thread (512 threads, 32 rows)
+        const int row = tid >> 4, seg = tid & 15;
+        const int ir = i0 + row;
+        if (ir >= N) return;
+        float L = 0.f;
+#pragma unroll
+        for (int w = 0; w < 8; ++w) L += xl[w * 32 + row];
+        const float inv = 1.f / L;
+        const float *src = acc_sh + row * C::APITCH + seg * SEG;
+        char *orow = p.o.ptr + b * p.o.sb + (int64_t)ir * p.o.sn + h * p.o.sh + seg * SEG * 2;
+        char *rrow = p.o_lo.ptr ? p.o_lo.ptr + b * p.o_lo.sb + (int64_t)ir * p.o_lo.sn + h * p.o_lo.sh + seg * SEG * 2 : nullptr;
+        float o[SEG];
+#pragma unroll
+        for (int x = 0; x < SEG; x += 4) {
+            float4 v = *reinterpret_cast<const float4 *>(src + x);
+            o[x] = v.x * inv;
+            o[x + 1] = v.y * inv;
+            o[x + 2] = v.z * inv;
+            o[x + 3] = v.w * inv;
+        }
+        if constexpr (SEG == 8) {
+            u32x4 ov, rv;
+#pragma unroll
+            for (int w = 0; w < 4; ++w) {
+                ov[w] = pack_bf16(o[2 * w], o[2 * w + 1]);
+                rv[w] = pack_bf16(o[2 * w] - bf16_lo(ov[w]), o[2 * w + 1] - bf16_hi(ov[w]));
+            }
+            st_global16(orow, ov);
+            if (rrow) st_global16(rrow, rv);
+        } else {
+            u32x2 ov, rv;
+#pragma unroll
+            for (int w = 0; w < 2; ++w) {
+                ov[w] = pack_bf16(o[2 * w], o[2 * w + 1]);
+                rv[w] = pack_bf16(o[2 * w] - bf16_lo(ov[w]), o[2 * w + 1] - bf16_hi(ov[w]));
+            }
+            *reinterpret_cast<u32x2 *>(orow) = ov;
+            if (rrow) *reinterpret_cast<u32x2 *>(rrow) = rv;
+        }
+        if (seg == 0) p.lse[((int64_t)b * p.H + h) * N + ir] = (xm[row] + __builtin_amdgcn_logf(L)) * kLn2;
+    }
+}
+
+}  // namespace sa2
