@@ -12,8 +12,7 @@
 
 #include "sa2_bwd.hpp"
 #include "sa2_bwd_kv8.hpp"
-#include "sa2_bwd_q8.hpp"
-#include "sa2_bwd_qk2.hpp"
+#include "sa2_bwd_q.hpp"
 #include "sa2_common.hpp"
 #include "sa2_lds.hpp"
 #include "sa2_qkv_norm.hpp"
@@ -40,7 +39,6 @@ int check_problem(const sa2_problem *p) {
     if (p->heads % p->kv_heads != 0)
         return fail(SA2_ERR_BAD_SHAPE, "heads=%d is not a multiple of kv_heads=%d", p->heads, p->kv_heads);
     if (p->w1 < 1 || p->w2 < 1) return fail(SA2_ERR_BAD_SHAPE, "windows w1=%d w2=%d must be >= 1", p->w1, p->w2);
-    if (p->w2 > 64) return fail(SA2_ERR_UNSUPPORTED, "w2=%d is not supported (at most 64)", p->w2);
     if (p->causal != 1) return fail(SA2_ERR_UNSUPPORTED, "only causal=1 is defined for the sliding windows");
     if (p->dtype != SA2_BF16) return fail(SA2_ERR_UNSUPPORTED, "dtype %d is not supported (bf16 only)", p->dtype);
     if (p->dim_head != 64 && p->dim_head != 128)
@@ -132,7 +130,7 @@ int sa2_version(void) { return SA2_VERSION; }
 const char *sa2_last_error(void) { return g_err; }
 
 int sa2_supported(int32_t dim_head, int32_t w1, int32_t w2, int32_t dtype) {
-    return (dim_head == 64 || dim_head == 128) && w1 >= 1 && w2 >= 1 && w2 <= 64 && dtype == SA2_BF16;
+    return (dim_head == 64 || dim_head == 128) && w1 >= 1 && w2 >= 1 && dtype == SA2_BF16;
 }
 
 static int check_saved(const sa2_saved *saved) {
@@ -246,13 +244,12 @@ static int bwd_pass_filter() {
     return 0;
 }
 
-// rows of K2/V2 a 32-row query tile can reach: 32 own + (w2max - 1) below it
-static int qk2_w2max(int w2) { return w2 <= 32 ? 32 : 64; }
+// rows below a 32-row query tile that its offsets reach (offsets run in rounds of eight)
+static int q_halo(int w2) { return 8 * ((w2 + 7) / 8) - 1; }
 
 int64_t sa2_bwd_workspace_bytes(const sa2_problem *prob) {
     if (check_problem(prob) != SA2_OK) return -1;
-    const int srows = 31 + qk2_w2max(prob->w2);
-    return sa2::qk2_ws_floats(prob->batch, prob->heads, prob->seq_len, prob->dim_head, srows) * 4;
+    return sa2::qk2_ws_floats(prob->batch, prob->heads, prob->seq_len, prob->dim_head, 32 + q_halo(prob->w2)) * 4;
 }
 
 int sa2_bwd_dq_dkv2(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
@@ -276,35 +273,25 @@ int sa2_bwd_dq_dkv2(const sa2_problem *prob, const sa2_tensor *q, const sa2_tens
     float *ws = static_cast<float *>(workspace);
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
     const int grid = prob->batch * prob->heads * ((prob->seq_len + 31) / 32);
-    const int w2max = qk2_w2max(prob->w2);
-    // offsets up to 32: two eight-wave passes (dq + dk2, then dv2); wider second windows take the
-    // fused four-wave kernel
-    const bool fused = w2max > 32;
+    const int halo = q_halo(prob->w2);
     const int pass = bwd_pass_filter();
     // with the forward's saved per-offset T the dv2 pass (a recomputation of S and T) is
     // replaced by a kernel that streams T once
-    const bool use_saved = saved != nullptr && !fused;
+    const bool use_saved = saved != nullptr;
     if (saved) {
         SA2_TRY(check_saved(saved));
         k.t_save = static_cast<char *>(saved->t);
         k.m_save = saved->m;
     }
-    if (!fused && prob->dim_head == 128) {
-        hipLaunchKernelGGL((sa2::bwd_q8_kernel<128, true>), dim3(grid), dim3(512), 0, s, k, ws);
-        if (pass != 1 && !use_saved) hipLaunchKernelGGL((sa2::bwd_q8_kernel<128, false>), dim3(grid), dim3(512), 0, s, k, ws);
-    } else if (!fused) {
-        hipLaunchKernelGGL((sa2::bwd_q8_kernel<64, true>), dim3(grid), dim3(512), 0, s, k, ws);
-        if (pass != 1 && !use_saved) hipLaunchKernelGGL((sa2::bwd_q8_kernel<64, false>), dim3(grid), dim3(512), 0, s, k, ws);
-    } else if (prob->dim_head == 128 && w2max == 32)
-        hipLaunchKernelGGL((sa2::bwd_qk2_kernel<128, 32>), dim3(grid), dim3(256), 0, s, k, ws);
-    else if (prob->dim_head == 128)
-        hipLaunchKernelGGL((sa2::bwd_qk2_kernel<128, 64>), dim3(grid), dim3(256), 0, s, k, ws);
-    else if (w2max == 32)
-        hipLaunchKernelGGL((sa2::bwd_qk2_kernel<64, 32>), dim3(grid), dim3(256), 0, s, k, ws);
-    else
-        hipLaunchKernelGGL((sa2::bwd_qk2_kernel<64, 64>), dim3(grid), dim3(256), 0, s, k, ws);
+    if (prob->dim_head == 128) {
+        hipLaunchKernelGGL((sa2::bwd_q_kernel<128, true>), dim3(grid), dim3(512), 0, s, k, ws, halo);
+        if (pass != 1 && !use_saved) hipLaunchKernelGGL((sa2::bwd_q_kernel<128, false>), dim3(grid), dim3(512), 0, s, k, ws, halo);
+    } else {
+        hipLaunchKernelGGL((sa2::bwd_q_kernel<64, true>), dim3(grid), dim3(512), 0, s, k, ws, halo);
+        if (pass != 1 && !use_saved) hipLaunchKernelGGL((sa2::bwd_q_kernel<64, false>), dim3(grid), dim3(512), 0, s, k, ws, halo);
+    }
     SA2_TRY(after_launch("dq/dk2/dv2"));
-    if (!fused && pass == 1) return SA2_OK;    // profiling one pass: leave the reductions out of its timing
+    if (pass == 1) return SA2_OK;    // profiling build, one pass: leave the reductions out of its timing
     if (use_saved) {
         const int rpb = 256 / (prob->dim_head / 8);
         const int dgrid = prob->batch * prob->kv_heads * ((prob->seq_len + rpb - 1) / rpb);
@@ -319,9 +306,9 @@ int sa2_bwd_dq_dkv2(const sa2_problem *prob, const sa2_tensor *q, const sa2_tens
     const int cgrid = (int)((rows + rows_per_block - 1) / rows_per_block);
     const int with_dv2 = use_saved ? 0 : 1;
     if (prob->dim_head == 128)
-        hipLaunchKernelGGL(sa2::dk2_dv2_combine_kernel<128>, dim3(cgrid), dim3(256), 0, s, k, ws, 31 + w2max, with_dv2);
+        hipLaunchKernelGGL(sa2::dk2_dv2_combine_kernel<128>, dim3(cgrid), dim3(256), 0, s, k, ws, 32 + halo, with_dv2);
     else
-        hipLaunchKernelGGL(sa2::dk2_dv2_combine_kernel<64>, dim3(cgrid), dim3(256), 0, s, k, ws, 31 + w2max, with_dv2);
+        hipLaunchKernelGGL(sa2::dk2_dv2_combine_kernel<64>, dim3(cgrid), dim3(256), 0, s, k, ws, 32 + halo, with_dv2);
     return after_launch("dk2/dv2 combine");
 }
 
@@ -336,16 +323,11 @@ int sa2_bwd_dkv1(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor 
     k.dv1 = dev(dv1);
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
     int grid = prob->batch * prob->kv_heads * ((prob->seq_len + 127) / 128);
-    // offsets up to 32: one eight-wave kernel for both outputs; wider second windows take the
-    // fused four-wave kernel
-    if (prob->w2 <= 32 && prob->dim_head == 128)
+    // dim_head 128: the two waves of a slab split the contractions; dim_head 64: each wave forms both outputs
+    if (prob->dim_head == 128)
         hipLaunchKernelGGL((sa2::bwd_kv8_kernel<128, sa2::kKvSplit>), dim3(grid), dim3(512), 0, s, k);
-    else if (prob->w2 <= 32)
-        hipLaunchKernelGGL((sa2::bwd_kv8_kernel<64, sa2::kKvBoth>), dim3(grid), dim3(512), 0, s, k);
-    else if (prob->dim_head == 128)
-        hipLaunchKernelGGL(sa2::bwd_dkv1_kernel<128>, dim3(grid), dim3(256), 0, s, k);
     else
-        hipLaunchKernelGGL(sa2::bwd_dkv1_kernel<64>, dim3(grid), dim3(256), 0, s, k);
+        hipLaunchKernelGGL((sa2::bwd_kv8_kernel<64, sa2::kKvBoth>), dim3(grid), dim3(512), 0, s, k);
     return after_launch("dk1/dv1");
 }
 

@@ -5,7 +5,8 @@
 // offset dlt); a pair holds the offsets 2m and 2m+1 of one query tile.  The q/do rows of a
 // query tile and the 63 k2/v2 rows its offsets (at most 32) can reach are staged in LDS
 // once per tile; from them the 512 threads build A = q*k2 and B = do*v2 of both steps
-// once per pair.  With P = exp2(S scale log2e - lse):
+// once per pair (A carries scale log2(e), so S is the exponent's variable part and dK1 comes out
+// times scale log2(e): it is stored times ln 2).  With P = exp2(S - lse log2(e)):
 //   S = A K1^T,  dP = B V1^T,  dS = P (dP - delta),  dK1^T += A^T dS,  dV1^T += B^T P.
 // One wave cannot overlap its own MFMA and VALU work, so every variant keeps two waves per
 // SIMD (at most 256 registers per wave):
@@ -153,22 +154,33 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     using ASwz = std::integral_constant<bool, L::A_SWZ>;
     using BSwz = std::integral_constant<bool, L::B_SWZ>;
 
-    // ---- pair iterator (g, it, m): offsets 2m and 2m+1 of query tile `it`, query head g of the group
+    // ---- pair iterator (g, it, blk, m): offsets 32 blk + 2m and 32 blk + 2m + 1 of query tile `it`, query head g
+    // of the group.  (it, blk) is the staging unit: the q/do rows of the tile and the 63 k2/v2 rows that the 32
+    // offsets of the block reach.
     struct Pair {
-        int g, it, m;
+        int g, it, blk, m;
     };
-    auto dmax_of = [&](int it) { return (p.w2 - 1 < 32 * it + 31) ? p.w2 - 1 : 32 * it + 31; };
-    auto next_pair = [&](Pair &s) {
-        if (2 * (++s.m) > dmax_of(s.it)) {
-            s.m = 0;
+    auto dtop_of = [&](int it) { return (p.w2 - 1 < 32 * it + 31) ? p.w2 - 1 : 32 * it + 31; };   // largest offset of a tile
+    auto dmax_of = [&](int it, int blk) {                 // largest offset of a block, relative to the block
+        const int d = dtop_of(it) - 32 * blk;
+        return d < 31 ? d : 31;
+    };
+    auto next_unit = [&](Pair &s) {      // first pair of the next (query head, query tile, offset block)
+        s.m = 0;
+        if (32 * (++s.blk) > dtop_of(s.it)) {
+            s.blk = 0;
             if (++s.it > it_end) {
                 s.it = it_begin;
                 ++s.g;
             }
         }
     };
+    auto next_pair = [&](Pair &s) {
+        if (2 * (++s.m) > dmax_of(s.it, s.blk)) next_unit(s);
+    };
     int npairs = 0;
-    for (int it = it_begin; it <= it_end; ++it) npairs += dmax_of(it) / 2 + 1;
+    for (int it = it_begin; it <= it_end; ++it)
+        for (int blk = 0; 32 * blk <= dtop_of(it); ++blk) npairs += dmax_of(it, blk) / 2 + 1;
     npairs *= p.G;
 
     // ---- row staging: per (query head, query tile) the q/do rows and the k2/v2 rows go
@@ -191,7 +203,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                 src = (row < 32 ? qg + (int64_t)i * p.q.sn : dog + (int64_t)i * p.dout.sn);
             } else {
                 const int rk = row - 64;
-                int kr = 32 * s.it - L::HALO + (rk < L::KROWS ? rk : rk - L::KROWS);
+                int kr = 32 * (s.it - s.blk) - L::HALO + (rk < L::KROWS ? rk : rk - L::KROWS);
                 kr = kr < 0 ? 0 : (kr < N ? kr : N - 1);
                 src = (rk < L::KROWS ? k2g + (int64_t)kr * p.k2.sn : v2g + (int64_t)kr * p.v2.sn);
             }
@@ -234,20 +246,20 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
         const u32x4 fo = ld_lds16(lds + L::DOS + row * L::RP + col);
 #pragma unroll
         for (int w = 0; w < 4; ++w) {
-            qx[2 * w] = bf16_lo(fq[w]);
-            qx[2 * w + 1] = bf16_hi(fq[w]);
+            qx[2 * w] = bf16_lo(fq[w]) * c2;
+            qx[2 * w + 1] = bf16_hi(fq[w]) * c2;
             ox[2 * w] = bf16_lo(fo[w]);
             ox[2 * w + 1] = bf16_hi(fo[w]);
         }
     };
     auto build = [&](const Pair &s, int buf) {
         const int row = b_row, col = b_col;
-        const int dmax = dmax_of(s.it);
+        const int dmax = dmax_of(s.it, s.blk);
         char *stage = lds + buf * L::PAIR;
         const int dl0 = 2 * s.m;                                   // never dead
         const bool dead1 = dl0 + 1 > dmax;
         const int dl1 = dead1 ? dl0 : dl0 + 1;
-        auto product = [&](const float (&xv)[8], int bs, auto is_a) {   // xv: q or dO piece, bs: k2 or v2 rows
+        auto product = [&](const float (&xv)[8], int bs, auto is_a) {   // xv: q (times scale log2 e) or dO piece, bs: k2 or v2 rows
             constexpr bool IS_A = decltype(is_a)::value;
             u32x4 r0, r1;
             const u32x4 f0 = ld_lds16(lds + bs + (row - dl0 + L::HALO) * L::RP + col);
@@ -267,21 +279,21 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
             product(ox, L::V2S, std::false_type{});
         } else {
             float xv[8];
-            auto unpack = [&](int xs) {
+            auto unpack = [&](int xs, float f) {
                 const u32x4 fx = ld_lds16(lds + xs + row * L::RP + col);
 #pragma unroll
                 for (int w = 0; w < 4; ++w) {
-                    xv[2 * w] = bf16_lo(fx[w]);
-                    xv[2 * w + 1] = bf16_hi(fx[w]);
+                    xv[2 * w] = bf16_lo(fx[w]) * f;
+                    xv[2 * w + 1] = bf16_hi(fx[w]) * f;
                 }
             };
             if (BOTH || tid < PIECES) {
-                unpack(L::QS);
+                unpack(L::QS, c2);
                 product(xv, L::K2S, std::true_type{});
             }
             if constexpr (BOTH) __builtin_amdgcn_sched_barrier(0);   // one product at a time: the dk1 pass has no registers for both
             if (BOTH || tid >= PIECES) {
-                unpack(L::DOS);
+                unpack(L::DOS, 1.f);
                 product(xv, L::V2S, std::false_type{});
             }
         }
@@ -289,25 +301,18 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
             const int e = tid >> 5, r = tid & 31;
             const int i = 32 * s.it + r;
             const int dlt = dl0 + e;
-            const bool valid = dlt <= dmax && i < N && i - dlt >= 0;
+            const bool valid = dlt <= dmax && i < N && i - 32 * s.blk - dlt >= 0;
             char *st = stage + e * L::STEP;
-            reinterpret_cast<float *>(st + L::LSE)[r] = valid ? reinterpret_cast<const float *>(lds + L::LSES)[r] : INFINITY;
+            // (negated: the logit chains start from it)
+            reinterpret_cast<float *>(st + L::LSE)[r] = valid ? -reinterpret_cast<const float *>(lds + L::LSES)[r] : -INFINITY;
             if constexpr (DK) reinterpret_cast<float *>(st + L::DEL)[r] = valid ? -reinterpret_cast<const float *>(lds + L::LSES)[32 + r] : 0.f;
         }
     };
-    auto next_tile = [&](Pair &s) {      // first pair of the next (query head, query tile)
-        s.m = 0;
-        if (++s.it > it_end) {
-            s.it = it_begin;
-            ++s.g;
-        }
-    };
-
-    Pair nb = {0, it_begin, 0};   // next pair to build
-    Pair cur = {0, it_begin, 0};  // pair being computed
-    Pair rw = {0, it_begin, 0};   // query tile whose rows are loaded next
+    Pair nb = {0, it_begin, 0, 0};   // next pair to build
+    Pair cur = {0, it_begin, 0, 0};  // pair being computed
+    Pair rw = {0, it_begin, 0, 0};   // staging unit whose rows are loaded next
     issue_rows(rw);
-    next_tile(rw);
+    next_unit(rw);
     write_rows();
     if (rw.g < p.G) issue_rows(rw);
     __syncthreads();
@@ -324,7 +329,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
             __syncthreads();                                    // the tiles of the pair are complete
             if (more && nb.m == 0) {
                 write_rows();
-                next_tile(rw);
+                next_unit(rw);
                 if (rw.g < p.G) issue_rows(rw);
                 __syncthreads();
             }
@@ -344,17 +349,19 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
 #pragma unroll
                     for (int e = 0; e < 2; ++e) {
                         const char *buf = pair + e * L::STEP;
-                        f32x16 X = zero16();
-#pragma unroll
-                        for (int kk = 0; kk < KS; ++kk) X = mfma32(swz_lane.row_frag(buf + L::AS, kk), k1f[kk], X);
+                        // the chain starts from -lse_i log2(e) (stored negated by the build; -inf for dead rows), and A
+                        // carries scale * log2(e): the result is the exponent
+                        f32x16 X;
 #pragma unroll
                         for (int a4 = 0; a4 < 4; ++a4) {
                             const float4 l4 = *reinterpret_cast<const float4 *>(buf + L::LSE + (8 * a4 + 4 * hf) * 4);
-                            X[4 * a4] = X[4 * a4] * c2 - l4.x;
-                            X[4 * a4 + 1] = X[4 * a4 + 1] * c2 - l4.y;
-                            X[4 * a4 + 2] = X[4 * a4 + 2] * c2 - l4.z;
-                            X[4 * a4 + 3] = X[4 * a4 + 3] * c2 - l4.w;
+                            X[4 * a4] = l4.x;
+                            X[4 * a4 + 1] = l4.y;
+                            X[4 * a4 + 2] = l4.z;
+                            X[4 * a4 + 3] = l4.w;
                         }
+#pragma unroll
+                        for (int kk = 0; kk < KS; ++kk) X = mfma32(swz_lane.row_frag(buf + L::AS, kk), k1f[kk], X);
                         if (!full) {
                             const int base = 32 * it + 4 * hf - j;   // i - j for register 0
 #pragma unroll
@@ -451,7 +458,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                     }
                 }
             }
-            if (j_ok) store_row<DT>(p.dk1.ptr + b * p.dk1.sb + (int64_t)j * p.dk1.sn + hk * p.dk1.sh + 16 * hf * 2, acc, p.scale);
+            if (j_ok) store_row<DT>(p.dk1.ptr + b * p.dk1.sb + (int64_t)j * p.dk1.sn + hk * p.dk1.sh + 16 * hf * 2, acc, kLn2);   // A carried scale log2(e)
         }
         return;
     }
@@ -463,7 +470,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                 // the next pair opens a new query tile: its rows replace the staged ones
                 // (all builds from the old rows ended before the barrier above)
                 write_rows();
-                next_tile(rw);
+                next_unit(rw);
                 if (rw.g < p.G) issue_rows(rw);
                 __syncthreads();
                 if constexpr (KEEP) unpack_own();
@@ -477,7 +484,17 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
         if (!wave_active || it < wit_lo || it > wit_hi) continue;
 
         // ---- S[i,j] (and dP[i,j]): rows = query rows of the tile, column = j
-        f32x16 X = zero16();
+        // the chain starts from -lse_i log2(e) (stored negated by the build; -inf for dead rows), and A carries
+        // scale * log2(e): the result is the exponent
+        f32x16 X;
+#pragma unroll
+        for (int a4 = 0; a4 < 4; ++a4) {
+            const float4 l4 = *reinterpret_cast<const float4 *>(buf + L::LSE + (8 * a4 + 4 * hf) * 4);
+            X[4 * a4] = l4.x;
+            X[4 * a4 + 1] = l4.y;
+            X[4 * a4 + 2] = l4.z;
+            X[4 * a4 + 3] = l4.w;
+        }
 #pragma unroll
         for (int kk = 0; kk < KS; ++kk) X = mfma32(row_frag(buf + L::AS, ASwz{}, kk), k1f[kk], X);
         f32x16 dP;
@@ -494,14 +511,6 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
             }
 #pragma unroll
             for (int kk = 0; kk < KS; ++kk) dP = mfma32(row_frag(buf + L::BS, BSwz{}, kk), v1f[kk], dP);
-        }
-#pragma unroll
-        for (int a4 = 0; a4 < 4; ++a4) {
-            const float4 l4 = *reinterpret_cast<const float4 *>(buf + L::LSE + (8 * a4 + 4 * hf) * 4);
-            X[4 * a4] = X[4 * a4] * c2 - l4.x;
-            X[4 * a4 + 1] = X[4 * a4 + 1] * c2 - l4.y;
-            X[4 * a4 + 2] = X[4 * a4 + 2] * c2 - l4.z;
-            X[4 * a4 + 3] = X[4 * a4 + 3] * c2 - l4.w;
         }
         const bool full = (jw + 31 <= 32 * it) && (jw + p.w1 > 32 * it + 31);
         if (!full) {
@@ -567,7 +576,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     collect(acc, red);
     char *dk1row = p.dk1.ptr + b * p.dk1.sb + (int64_t)j * p.dk1.sn + hk * p.dk1.sh + 16 * hf * 2;
     char *dv1row = p.dv1.ptr + b * p.dv1.sb + (int64_t)j * p.dv1.sn + hk * p.dv1.sh + 16 * hf * 2;
-    if constexpr (DK) store_row<DT>(dk1row, acc, p.scale);
+    if constexpr (DK) store_row<DT>(dk1row, acc, kLn2);   // A carried scale log2(e)
     if constexpr (MODE == kKvDv) store_row<DT>(dv1row, acc, 1.f);
     if constexpr (TWO) {
         collect(acc2, red + L::RED / 4);

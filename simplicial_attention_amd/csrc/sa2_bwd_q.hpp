@@ -1,0 +1,499 @@
+// Backward kernels that own query rows: dQ and dK2 (pass DQ), dV2 by recomputation (pass DV).
+//
+// Same shape as the forward: one workgroup owns 32 query rows i of one (batch, head), in round r
+// wave w handles the offset dlt = i - k = 8r + w (any second window), and all waves walk the same
+// K1/V1 tiles through a double-buffered LDS ring, one tile and one barrier per step.  A fused
+// kernel (S, dP, T and G accumulators together) needs more than 256 registers per wave, which
+// forces one wave per SIMD; so the work is split into two passes that each fit two waves per SIMD:
+//
+//   pass DQ, with A = q_i * k2_{i-dlt} * scale * log2(e), B = do_i * v2_{i-dlt}:
+//       S^T = K1 A^T,  dP^T = V1 B^T,  dS = P (dP - delta_i),  G^T += K1^T dS^T
+//       dq_i += k2_{i-dlt} * G_i,   dk2_{i-dlt} += q_i * G_i
+//   pass DV:
+//       S^T = K1 A^T,  T^T += V1^T P^T,   dv2_{i-dlt} += do_i * T_i
+//
+// with P = exp2(S - lse_i log2(e)).  The logit chain starts from -lse_i log2(e) (from -inf in lanes
+// without a valid (row, offset)) plus an additive 0 / -inf mask from an LDS table on the diagonal tile
+// and on the tiles that the window's lower edge crosses, so its result is the exponent; the dP chain
+// starts from -delta_i.  No mask, subtraction or scaling code follows the chains.
+// Sums over offsets go to fp32 LDS rows shared by the workgroup; a round's additions run in eight
+// barrier-separated phases in which wave w owns the d-slice (w + phase) mod 8, so no two waves touch
+// one element at a time and the order is fixed (bitwise reproducible, no atomics).  The rows k that
+// the offsets scatter to live in a 64-row circular buffer (row k in slot (k - i0) mod 64); the eight
+// rows that a round completes go to the fp32 workspace that dk2_dv2_combine_kernel reduces:
+// [tensor 0: dk2, 1: dv2][b][h][tile][32 + halo][D], row x of a tile <-> k = i0 - halo + x, with
+// halo = 8 ceil(w2 / 8) - 1.
+#pragma once
+
+#include <type_traits>
+
+#include "sa2_common.hpp"
+#include "sa2_lds.hpp"
+
+namespace sa2 {
+
+template <int D, bool DQ>
+struct QCfg {
+    static constexpr int KS = D / 16;
+    static constexpr int DT = D / 32;
+    static constexpr int PITCH = tile_pitch<D>();
+    static constexpr int TILE = 32 * PITCH;           // a tile read row-major
+    static constexpr int TPITCH = tr_pitch<D>();
+    static constexpr int TRT = 32 * TPITCH;           // a tile read through transposed reads
+    // ring buffer: DQ: [K1, read both ways: swizzled layout of sa2_lds.hpp][V1 row-major];  DV: [K1 row-major][V1 transposed-read]
+    static constexpr int OFF_TR = DQ ? 0 : TILE;      // the tile read through transposed reads
+    static constexpr int OFF_V = TRT;                 // DQ only
+    static constexpr int BUF = TILE + TRT;
+    static constexpr int RING = 2 * BUF;
+    static constexpr int SPITCH = D + 4;              // floats per row of the fp32 rows
+    static constexpr int DQS = RING;                  // dq rows [32][SPITCH]            (DQ only)
+    static constexpr int SC = RING + (DQ ? 32 * SPITCH * 4 : 0);   // scatter rows, circular [64][SPITCH]
+    static constexpr int QS = SC + 64 * SPITCH * 4;                // q rows   [32][PITCH]
+    static constexpr int DOS = QS + TILE;                          // do rows  [32][PITCH]
+    static constexpr int K2S = DOS + TILE;                         // k2 rows, circular [64][PITCH]
+    static constexpr int V2S = K2S + 64 * PITCH;                   // v2 rows, circular [64][PITCH]  (DQ only)
+    static constexpr int MASKS = DQ ? V2S + 64 * PITCH : V2S;      // additive masks, 3 tables [4 quarters][64 lanes][4 floats]
+    static constexpr int MASK = 16 * 64 * 4;
+    static constexpr int LDS = MASKS + 3 * MASK;
+    static constexpr int PPR = D / 8;                 // 16-byte pieces per row
+    static constexpr int PIECES = 32 * PPR;           // ... per tile
+};
+
+// workspace layout (floats): [tensor 0: dk2, 1: dv2][b][h][tile][srows][D], srows = 32 + halo
+__host__ __device__ inline int64_t qk2_ws_floats(int B, int H, int N, int D, int srows) {
+    return 2ll * B * H * ((N + 31) / 32) * srows * D;
+}
+
+template <int NS, typename F>
+__device__ __forceinline__ void with_slice(int s, F &&f) {
+    static_assert(NS == 4 || NS == 8, "slice count");
+    if constexpr (NS == 8) {
+        switch (s & 7) {
+            case 0: f(std::integral_constant<int, 0>{}); break;
+            case 1: f(std::integral_constant<int, 1>{}); break;
+            case 2: f(std::integral_constant<int, 2>{}); break;
+            case 3: f(std::integral_constant<int, 3>{}); break;
+            case 4: f(std::integral_constant<int, 4>{}); break;
+            case 5: f(std::integral_constant<int, 5>{}); break;
+            case 6: f(std::integral_constant<int, 6>{}); break;
+            default: f(std::integral_constant<int, 7>{}); break;
+        }
+    } else {
+        switch (s & 3) {
+            case 0: f(std::integral_constant<int, 0>{}); break;
+            case 1: f(std::integral_constant<int, 1>{}); break;
+            case 2: f(std::integral_constant<int, 2>{}); break;
+            default: f(std::integral_constant<int, 3>{}); break;
+        }
+    }
+}
+
+template <int D, bool DQ>
+__global__ __launch_bounds__(512) void bwd_q_kernel(KParams p, float *ws, int halo) {
+    using C = QCfg<D, DQ>;
+    constexpr int KS = C::KS, DT = C::DT, PPR = C::PPR, PITCH = C::PITCH;
+    __shared__ __attribute__((aligned(16))) char lds[C::LDS];
+
+    const int N = p.N;
+    const int ntile = (N + 31) / 32;
+    const int item = xcd_contiguous(blockIdx.x, gridDim.x);
+    const int tile = ntile - 1 - item % ntile;
+    const int bh = item / ntile;
+    const int h = bh % p.H, b = bh / p.H;
+    const int hk = h / p.G;
+
+    const int tid = threadIdx.x;
+    const int wave = wave_index(), lane = tid & 63;
+    const int c = lane & 31, hf = lane >> 5;
+    const int i0 = tile * 32;
+    const int i = i0 + c;
+    const bool row_ok = i < N;
+    const int ic = row_ok ? i : N - 1;
+
+    const char *k1g = p.k1.ptr + b * p.k1.sb + hk * p.k1.sh;
+    const char *v1g = p.v1.ptr + b * p.v1.sb + hk * p.v1.sh;
+    const char *k2g = p.k2.ptr + b * p.k2.sb + hk * p.k2.sh;
+    const char *v2g = p.v2.ptr + b * p.v2.sb + hk * p.v2.sh;
+    const float lse2 = p.lse[((int64_t)b * p.H + h) * N + ic] * kLog2e;
+    float dl = 0.f;
+    if constexpr (DQ) dl = p.delta[((int64_t)b * p.H + h) * N + ic];
+
+    // tiles of the first window, walked in order t_lo .. t_hi; masked: the tiles below mid_lo and the diagonal one
+    const int t_lo = (i0 - p.w1 + 1 > 0 ? i0 - p.w1 + 1 : 0) / 32;
+    const int t_hi = i0 / 32;
+    const int NT = t_hi - t_lo + 1;
+    int mid_lo = (i0 + 31 - p.w1 >= 0) ? (i0 + 31 - p.w1) / 32 + 1 : t_lo;   // first tile that no row masks at the window's lower edge
+    mid_lo = mid_lo > t_hi ? t_hi : mid_lo;
+    const int n_head = mid_lo - t_lo;                 // leading steps of a round with a lower-edge mask (at most 2)
+    const int nd = p.w2 < i0 + 32 ? p.w2 : i0 + 32;   // offsets that meet at least one valid k
+    const int R = (nd + 7) / 8;
+    const int U = R * NT;
+
+    // ---- ring staging: the first PIECES threads move one 16-byte piece of K1 and of V1 per tile
+    const bool stager = tid < C::PIECES;
+    const int st_row = tid / PPR, st_col = (tid % PPR) * 16;
+    const int st_off_k = DQ ? swz_store_off<D>(st_row, st_col) : st_row * PITCH + st_col;
+    const int st_off_v = DQ ? C::OFF_V + st_row * PITCH + st_col : C::OFF_TR + st_row * C::TPITCH + st_col;
+    u32x4 st_k = {0u, 0u, 0u, 0u}, st_v = {0u, 0u, 0u, 0u};
+    int n_load = 0, u_load = 0;
+    // address = tile base (uniform) + this thread's row and column (32 bits); only the diagonal tile can
+    // reach past the last row, so only it needs a clamped row
+    const int st_row_diag = i0 + st_row < N ? st_row : N - 1 - i0;
+    const uint32_t so_k = (uint32_t)(st_row * (int)p.k1.sn + st_col), so_v = (uint32_t)(st_row * (int)p.v1.sn + st_col);
+    const uint32_t so_k_diag = (uint32_t)(st_row_diag * (int)p.k1.sn + st_col), so_v_diag = (uint32_t)(st_row_diag * (int)p.v1.sn + st_col);
+    auto issue_loads = [&]() {
+        const int t = t_lo + n_load;
+        const char *kb = k1g + (int64_t)(32 * t) * p.k1.sn;
+        const char *vb = v1g + (int64_t)(32 * t) * p.v1.sn;
+        if (stager) {
+            st_k = ld_global16(kb + (t == t_hi ? so_k_diag : so_k));
+            st_v = ld_global16(vb + (t == t_hi ? so_v_diag : so_v));
+        }
+        ++u_load;
+        n_load = (n_load == NT - 1) ? 0 : n_load + 1;
+    };
+    auto write_stage = [&](int buf_off) {
+        if (stager) {
+            *reinterpret_cast<u32x4 *>(lds + buf_off + st_off_k) = st_k;
+            *reinterpret_cast<u32x4 *>(lds + buf_off + st_off_v) = st_v;
+        }
+    };
+    const int r_lane = c * PITCH + 16 * hf;                              // row-major fragment: row c, pieces 2*kk + hf
+    const int t_lane = C::OFF_TR + tr_lane_off<D, C::TPITCH>(lane);      // transposed fragment, per-lane part
+    const SwzLane<D> swz_lane(lane);                                      // DQ: fragments of the swizzled K1 tile
+
+    // ---- fp32 rows shared by the workgroup, zeroed; q/do rows and the k2/v2 rows of the first round staged
+    float *dqs = reinterpret_cast<float *>(lds + C::DQS);
+    float *sc = reinterpret_cast<float *>(lds + C::SC);
+    {
+        float4 *z = reinterpret_cast<float4 *>(lds + C::RING);
+        constexpr int NZ = (C::QS - C::RING) / 16;
+        for (int x = tid; x < NZ; x += 512) z[x] = make_float4(0.f, 0.f, 0.f, 0.f);
+        const char *qg = p.q.ptr + b * p.q.sb + h * p.q.sh;
+        const char *dog = p.dout.ptr + b * p.dout.sb + h * p.dout.sh;
+        for (int x = tid; x < 32 * PPR; x += 512) {
+            const int row = x / PPR, col = (x % PPR) * 16;
+            int ii = i0 + row;
+            ii = ii < N ? ii : N - 1;
+            *reinterpret_cast<u32x4 *>(lds + C::QS + row * PITCH + col) = ld_global16(qg + (int64_t)ii * p.q.sn + col);
+            *reinterpret_cast<u32x4 *>(lds + C::DOS + row * PITCH + col) = ld_global16(dog + (int64_t)ii * p.dout.sn + col);
+        }
+        for (int x = tid; x < 39 * PPR; x += 512) {
+            const int row = x / PPR, col = (x % PPR) * 16;
+            int kk2 = i0 - 7 + row;
+            kk2 = kk2 < 0 ? 0 : (kk2 < N ? kk2 : N - 1);
+            const int slot = (row - 7) & 63;
+            *reinterpret_cast<u32x4 *>(lds + C::K2S + slot * PITCH + col) = ld_global16(k2g + (int64_t)kk2 * p.k2.sn + col);
+            if constexpr (DQ)
+                *reinterpret_cast<u32x4 *>(lds + C::V2S + slot * PITCH + col) = ld_global16(v2g + (int64_t)kk2 * p.v2.sn + col);
+        }
+    }
+    // additive masks: table 0 for the diagonal tile, tables 1, 2 for the tiles the lower window edge
+    // crosses.  Entry (lane, rr) is 0 if query row i0 + c attends key row 32 t + 4 hf + e(rr), else -inf
+    for (int x = tid; x < 3 * 256; x += 512) {
+        const int tab = x >> 8, qq = (x >> 6) & 3, ln = x & 63;
+        const int t = tab == 0 ? t_hi : t_lo + tab - 1;
+        const int rel = (ln & 31) + 32 * (t_hi - t) - 4 * (ln >> 5);
+        float4 m4;
+        float *mp = &m4.x;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) mp[e] = ((unsigned)(rel - (8 * qq + e)) < (unsigned)p.w1) ? 0.f : -INFINITY;
+        *reinterpret_cast<float4 *>(lds + C::MASKS + tab * C::MASK + qq * 1024 + ln * 16) = m4;
+    }
+    // the 8 k2 (and v2) rows that round r + 1 adds (k - i0 = -8r - 15 .. -8r - 8), one 16-byte piece per thread
+    const bool row_stager = tid < (DQ ? 2 : 1) * 8 * PPR;
+    const int rs_sel = tid / (8 * PPR), rs_row = (tid / PPR) % 8, rs_col = (tid % PPR) * 16;
+    u32x4 st_r = {0u, 0u, 0u, 0u};
+    auto issue_rows = [&](int r) {
+        if (row_stager) {
+            int kk2 = i0 - 8 * r - 15 + rs_row;
+            kk2 = kk2 < 0 ? 0 : (kk2 < N ? kk2 : N - 1);
+            st_r = ld_global16((rs_sel ? v2g + (int64_t)kk2 * p.v2.sn : k2g + (int64_t)kk2 * p.k2.sn) + rs_col);
+        }
+    };
+    auto write_rows = [&](int r) {
+        if (row_stager) {
+            const int slot = (-8 * r - 15 + rs_row) & 63;
+            *reinterpret_cast<u32x4 *>(lds + (rs_sel ? C::V2S : C::K2S) + slot * PITCH + rs_col) = st_r;
+        }
+    };
+    // scatter rows of this tile in the workspace: row x <-> k = i0 - halo + x
+    const int srows = 32 + halo;
+    const int64_t per_tensor = (int64_t)p.B * p.H * ntile * srows * D;
+    float *wk = ws + (DQ ? 0 : per_tensor) + (((int64_t)b * p.H + h) * ntile + tile) * srows * D;
+    // rows k - i0 = lo .. lo + n - 1 of the circular buffer go to the workspace and are cleared for reuse
+    auto flush_rows = [&](int lo, int n) {
+        for (int x = tid; x < n * (D / 4); x += 512) {
+            const int rel = lo + x / (D / 4), col = (x % (D / 4)) * 4;
+            float4 *src = reinterpret_cast<float4 *>(sc + ((rel & 63) * C::SPITCH + col));
+            *reinterpret_cast<float4 *>(wk + (int64_t)(rel + halo) * D + col) = *src;
+            *src = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    };
+
+    // ring protocol: step u lives in buffer u & 1; it is written at the end of step u - 1 (every wave
+    // has passed the barrier of step u - 1, so none still reads that buffer) from registers loaded
+    // one step earlier, and published by the barrier of step u
+    issue_loads();
+    write_stage(0);
+    if (U > 1) issue_loads();
+    int u = 0;
+    auto stage_ahead = [&]() {
+        if (u + 1 < U) {
+            write_stage(((u + 1) & 1) * C::BUF);
+            if (u_load < U) issue_loads();
+        }
+        ++u;
+    };
+
+    f32x16 neg_delta;          // DQ: -delta_i in every element (one query row per lane column)
+#pragma unroll
+    for (int rr = 0; rr < 16; ++rr) neg_delta[rr] = -dl;
+    f32x16 acc[DT];            // G^T (DQ) or T^T (DV) of the running offset
+    u32x4 A[KS];
+    u32x4 Bv[DQ ? KS : 1];
+
+    __syncthreads();
+    for (int r = 0; r < R; ++r) {
+        const int dlt = 8 * r + wave;
+        const int kr = i - dlt;
+        const bool col_ok = row_ok && kr >= 0 && dlt < p.w2;
+        const bool wave_on = wave_any(col_ok);
+        const int slot = (c - dlt) & 63;              // slot of row k = i - dlt in the circular rows
+        {
+            const char *qr = lds + C::QS + c * PITCH + 16 * hf;
+            const char *k2r = lds + C::K2S + slot * PITCH + 16 * hf;
+            const float c2 = p.scale_log2e;
+#pragma unroll
+            for (int kk = 0; kk < KS; ++kk) {
+                const u32x4 fq = ld_lds16(qr + 32 * kk), fk = ld_lds16(k2r + 32 * kk);
+#pragma unroll
+                for (int w = 0; w < 4; ++w)
+                    A[kk][w] = pack_bf16(bf16_lo(fq[w]) * bf16_lo(fk[w]) * c2, bf16_hi(fq[w]) * bf16_hi(fk[w]) * c2);
+            }
+            if constexpr (DQ) {
+                const char *dor = lds + C::DOS + c * PITCH + 16 * hf;
+                const char *v2r = lds + C::V2S + slot * PITCH + 16 * hf;
+#pragma unroll
+                for (int kk = 0; kk < KS; ++kk) Bv[kk] = mul_bf16x8(ld_lds16(dor + 32 * kk), ld_lds16(v2r + 32 * kk));
+            }
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) acc[dt] = zero16();
+        }
+        const float nl = col_ok ? -lse2 : -INFINITY;  // where the logit chains start
+
+        for (int n = 0; n < NT; ++n) {
+            __syncthreads();
+            if (wave_on) {
+                const char *sub = lds + (u & 1) * C::BUF;
+                const int t = t_lo + n;
+                f32x16 X;
+                if (t == t_hi || n < n_head) {
+                    const char *mk = lds + C::MASKS + (t == t_hi ? 0 : 1 + n) * C::MASK + lane * 16;
+#pragma unroll
+                    for (int qq = 0; qq < 4; ++qq) {
+                        const float4 m4 = *reinterpret_cast<const float4 *>(mk + qq * 1024);
+                        X[4 * qq] = m4.x + nl;
+                        X[4 * qq + 1] = m4.y + nl;
+                        X[4 * qq + 2] = m4.z + nl;
+                        X[4 * qq + 3] = m4.w + nl;
+                    }
+                } else {
+#pragma unroll
+                    for (int rr = 0; rr < 16; ++rr) X[rr] = nl;
+                }
+#pragma unroll
+                for (int kk = 0; kk < KS; ++kk) X = mfma32(DQ ? swz_lane.row_frag(sub, kk) : ld_lds16(sub + r_lane + 32 * kk), A[kk], X);
+                f32x16 dP;
+                if constexpr (DQ) {
+                    // the chain starts from a register set that holds -delta_i: dP - delta costs no VALU work
+                    dP = mfma32(ld_lds16(sub + C::OFF_V + r_lane), Bv[0], neg_delta);
+#pragma unroll
+                    for (int kk = 1; kk < KS; ++kk) dP = mfma32(ld_lds16(sub + C::OFF_V + r_lane + 32 * kk), Bv[kk], dP);
+                }
+                u32x4 pb[2];
+#pragma unroll
+                for (int rr = 0; rr < 16; rr += 2) {
+                    float p0 = fast_exp2(X[rr]);
+                    float p1 = fast_exp2(X[rr + 1]);
+                    if constexpr (DQ) {
+                        p0 *= dP[rr];
+                        p1 *= dP[rr + 1];
+                    }
+                    pb[rr >> 3][(rr & 7) >> 1] = pack_bf16(p0, p1);
+                }
+#pragma unroll
+                for (int k2s = 0; k2s < 2; ++k2s)
+#pragma unroll
+                    for (int dt = 0; dt < DT; ++dt) {
+                        u32x4 fr;
+                        if constexpr (DQ) {
+                            fr = swz_lane.tr_frag(sub, k2s, dt);
+                        } else {
+                            const u32x2 lo = lds_read_tr<D, C::TPITCH>(sub + t_lane, 16 * k2s, 32 * dt);
+                            const u32x2 hi = lds_read_tr<D, C::TPITCH>(sub + t_lane, 16 * k2s + 8, 32 * dt);
+                            fr = (u32x4){lo[0], lo[1], hi[0], hi[1]};
+                        }
+                        acc[dt] = mfma32(fr, pb[k2s], acc[dt]);
+                    }
+            }
+            stage_ahead();
+        }
+
+        // ---- round end: add into the shared fp32 rows, one d-slice per wave and phase
+        {
+            if (r + 1 < R) issue_rows(r);      // the rows that the next round adds arrive behind the phases below
+            const char *qr = lds + (DQ ? C::QS : C::DOS) + c * PITCH + 16 * hf * 2;   // factor of the scattered rows
+            const char *k2r = lds + C::K2S + slot * PITCH + 16 * hf * 2;
+            float *srow_p = sc + slot * C::SPITCH + 16 * hf;
+            float *drow_p = dqs + c * C::SPITCH + 16 * hf;
+            auto add_slice = [&](auto slice_tag) {
+                constexpr int S = decltype(slice_tag)::value;     // slice: dt = S / 2, registers 8*(S%2) .. +7
+                constexpr int dt = S >> 1, r0 = 8 * (S & 1);
+                const u32x4 xq = ld_lds16(qr + dt * 64 + r0 * 2);
+                float *dst = srow_p + 32 * dt + r0;
+                float4 a0 = *reinterpret_cast<float4 *>(dst), a1 = *reinterpret_cast<float4 *>(dst + 4);
+                a0.x += bf16_lo(xq[0]) * acc[dt][r0];
+                a0.y += bf16_hi(xq[0]) * acc[dt][r0 + 1];
+                a0.z += bf16_lo(xq[1]) * acc[dt][r0 + 2];
+                a0.w += bf16_hi(xq[1]) * acc[dt][r0 + 3];
+                a1.x += bf16_lo(xq[2]) * acc[dt][r0 + 4];
+                a1.y += bf16_hi(xq[2]) * acc[dt][r0 + 5];
+                a1.z += bf16_lo(xq[3]) * acc[dt][r0 + 6];
+                a1.w += bf16_hi(xq[3]) * acc[dt][r0 + 7];
+                *reinterpret_cast<float4 *>(dst) = a0;
+                *reinterpret_cast<float4 *>(dst + 4) = a1;
+                if constexpr (DQ) {
+                    const u32x4 xk = ld_lds16(k2r + dt * 64 + r0 * 2);
+                    float *dd = drow_p + 32 * dt + r0;
+                    float4 b0 = *reinterpret_cast<float4 *>(dd), b1 = *reinterpret_cast<float4 *>(dd + 4);
+                    b0.x += bf16_lo(xk[0]) * acc[dt][r0];
+                    b0.y += bf16_hi(xk[0]) * acc[dt][r0 + 1];
+                    b0.z += bf16_lo(xk[1]) * acc[dt][r0 + 2];
+                    b0.w += bf16_hi(xk[1]) * acc[dt][r0 + 3];
+                    b1.x += bf16_lo(xk[2]) * acc[dt][r0 + 4];
+                    b1.y += bf16_hi(xk[2]) * acc[dt][r0 + 5];
+                    b1.z += bf16_lo(xk[3]) * acc[dt][r0 + 6];
+                    b1.w += bf16_hi(xk[3]) * acc[dt][r0 + 7];
+                    *reinterpret_cast<float4 *>(dd) = b0;
+                    *reinterpret_cast<float4 *>(dd + 4) = b1;
+                }
+            };
+            for (int ph = 0; ph < 8; ++ph) {
+                // D = 128: eight slices.  D = 64: four slices; waves 0-3 use phases 0-3, waves 4-7 phases 4-7
+                if (DT == 4 || (ph >> 2) == (wave >> 2)) with_slice<2 * DT>(wave + ph, add_slice);
+                if (ph == 7 && r + 1 < R) write_rows(r);    // (their slots are not in use in this round)
+                __syncthreads();
+            }
+            // the rows k - i0 = 24 - 8r .. 31 - 8r are complete: no later round reaches them
+            if (r + 1 < R) flush_rows(24 - 8 * r, 8);
+        }
+    }
+    // ---- the rows that the last round leaves: k - i0 = -8 (R - 1) - 7 .. 31 - 8 (R - 1)
+    flush_rows(-8 * (R - 1) - 7, 39);
+
+    // ---- dq rows to global memory (bf16, scaled)
+    if constexpr (DQ) {
+        constexpr int SEG = D / 16;
+        const int row = tid >> 4, seg = tid & 15;
+        const int ir = i0 + row;
+        if (ir < N) {
+            const float *src = dqs + row * C::SPITCH + seg * SEG;
+            char *orow = p.dq.ptr + b * p.dq.sb + (int64_t)ir * p.dq.sn + h * p.dq.sh + seg * SEG * 2;
+            float4 a = *reinterpret_cast<const float4 *>(src);
+            if constexpr (SEG == 8) {
+                float4 bq = *reinterpret_cast<const float4 *>(src + 4);
+                u32x4 ov = {pack_bf16(a.x * p.scale, a.y * p.scale), pack_bf16(a.z * p.scale, a.w * p.scale),
+                            pack_bf16(bq.x * p.scale, bq.y * p.scale), pack_bf16(bq.z * p.scale, bq.w * p.scale)};
+                st_global16(orow, ov);
+            } else {
+                u32x2 ov = {pack_bf16(a.x * p.scale, a.y * p.scale), pack_bf16(a.z * p.scale, a.w * p.scale)};
+                *reinterpret_cast<u32x2 *>(orow) = ov;
+            }
+        }
+    }
+}
+
+// dV2 from the forward's saved per-offset T:
+//     dv2[b,k,hk,:] = sum_g sum_dlt do[b,k+dlt,h,:] * T[b,h,dlt,k+dlt,:] * 2^(m[b,h,dlt,k+dlt] - lse2[b,h,k+dlt])
+// (h = hk*G + g).  Streams T once from HBM; a thread owns 8 d of one row k.
+template <int D>
+__global__ __launch_bounds__(256) void dv2_from_saved_kernel(KParams p) {
+    constexpr int LP = D / 8;                 // threads per row
+    constexpr int RPB = 256 / LP;             // rows per block
+    const int N = p.N;
+    const int nblk = (N + RPB - 1) / RPB;
+    const int blk = blockIdx.x % nblk;
+    const int bh = blockIdx.x / nblk;
+    const int hk = bh % p.HK, b = bh / p.HK;
+    const int k = blk * RPB + threadIdx.x / LP;
+    const int col = (threadIdx.x % LP) * 16;  // byte offset inside a row
+    if (k >= N) return;
+    float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+    const int nd = p.w2 < N - k ? p.w2 : N - k;
+    for (int g = 0; g < p.G; ++g) {
+        const int h = hk * p.G + g;
+        const int64_t bh_row = ((int64_t)b * p.H + h);
+        const char *dog = p.dout.ptr + b * p.dout.sb + h * p.dout.sh + col;
+        const float *lse = p.lse + bh_row * N;
+#pragma unroll 8
+        for (int dlt = 0; dlt < nd; ++dlt) {
+            const int i = k + dlt;
+            const int64_t srow = (bh_row * p.w2 + dlt) * N + i;
+            const u32x4 t = ld_global16(p.t_save + srow * (D * 2) + col);
+            const u32x4 o = ld_global16(dog + (int64_t)i * p.dout.sn);
+            const float w = fast_exp2(p.m_save[srow] - lse[i] * kLog2e);
+#pragma unroll
+            for (int x = 0; x < 4; ++x) {
+                acc[2 * x] += bf16_lo(o[x]) * bf16_lo(t[x]) * w;
+                acc[2 * x + 1] += bf16_hi(o[x]) * bf16_hi(t[x]) * w;
+            }
+        }
+    }
+    u32x4 r = {pack_bf16(acc[0], acc[1]), pack_bf16(acc[2], acc[3]), pack_bf16(acc[4], acc[5]), pack_bf16(acc[6], acc[7])};
+    st_global16(p.dv2.ptr + b * p.dv2.sb + (int64_t)k * p.dv2.sn + hk * p.dv2.sh + col, r);
+}
+
+// dK2 / dV2 from the partial rows of the workspace: sums the tiles that reach a row and the query heads of a group.
+// Workspace rows of a tile with first query row i0: index x <-> k = i0 - halo + x, so
+// rows 0..halo-1 are the halo below the tile and rows halo..halo+31 its own rows.
+template <int D>
+__global__ __launch_bounds__(256) void dk2_dv2_combine_kernel(KParams p, const float *ws, int srows, int with_dv2) {
+    constexpr int LP = D / 8;   // threads per row, 8 d each
+    const int N = p.N, ntile = (N + 31) / 32;
+    const int halo = srows - 32;
+    const int64_t rows = (int64_t)p.B * p.HK * N;
+    const int64_t row = (int64_t)blockIdx.x * (256 / LP) + threadIdx.x / LP;
+    if (row >= rows) return;
+    const int piece = threadIdx.x % LP;
+    const int k = (int)(row % N);
+    const int hk = (int)((row / N) % p.HK);
+    const int b = (int)(row / ((int64_t)N * p.HK));
+    const int tile = k / 32, kl = k % 32;
+    const int64_t per_tensor = (int64_t)p.B * p.H * ntile * srows * D;
+    float ak[8], av[8];
+#pragma unroll
+    for (int x = 0; x < 8; ++x) ak[x] = av[x] = 0.f;
+    for (int g = 0; g < p.G; ++g) {
+        const int h = hk * p.G + g;
+        const float *base = ws + (((int64_t)b * p.H + h) * ntile) * srows * D;
+        for (int m = 0; tile + m < ntile && kl + halo - 32 * m >= 0; ++m) {
+            const float *src = base + ((int64_t)(tile + m) * srows + (kl + halo - 32 * m)) * D + piece * 8;
+#pragma unroll
+            for (int x = 0; x < 8; ++x) {
+                ak[x] += src[x];
+                if (with_dv2) av[x] += src[per_tensor + x];
+            }
+        }
+    }
+    u32x4 ok, ov;
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+        ok[w] = pack_bf16(ak[2 * w] * p.scale, ak[2 * w + 1] * p.scale);
+        ov[w] = pack_bf16(av[2 * w], av[2 * w + 1]);
+    }
+    st_global16(p.dk2.ptr + b * p.dk2.sb + (int64_t)k * p.dk2.sn + hk * p.dk2.sh + piece * 16, ok);
+    if (with_dv2) st_global16(p.dv2.ptr + b * p.dv2.sb + (int64_t)k * p.dv2.sn + hk * p.dv2.sh + piece * 16, ov);
+}
+
+}  // namespace sa2

@@ -79,7 +79,7 @@ class SlidingTwoSimplicialAttention(Function):
             raise ValueError('window sizes must be at least 1')
         lib = _native.load()
         if not lib.sa2_supported(dim, w1, w2, _native.SA2_BF16):
-            raise NotImplementedError(f'dim_head={dim}, w1={w1}, w2={w2} is not covered by the kernels (dim_head 64 or 128, w2 <= 64)')
+            raise NotImplementedError(f'dim_head={dim}, w1={w1}, w2={w2} is not covered by the kernels (dim_head 64 or 128)')
 
         q, k1, k2, v1, v2 = (_unit_inner_stride(t) for t in tensors)
         scale = dim ** -0.5 if scale is None else float(scale)
@@ -92,7 +92,7 @@ class SlidingTwoSimplicialAttention(Function):
         # per-offset value partials T (and their references), kept for the backward when
         # they fit the budget: dV2 then needs no recomputation of the attention weights
         t_save = m_save = None
-        if needs_grad and w2 <= 32 and 0 < lib.sa2_saved_t_bytes(prob) <= save_partials_max_bytes():
+        if needs_grad and 0 < lib.sa2_saved_t_bytes(prob) <= save_partials_max_bytes():
             t_save = torch.empty((batch, heads, w2, seq_len, dim), dtype=q.dtype, device=q.device)
             m_save = torch.empty((batch, heads, w2, seq_len), dtype=torch.float32, device=q.device)
         with torch.cuda.device_of(q):

@@ -5,6 +5,7 @@ Every shape runs with both input distributions and the tolerance stated for each
 import pytest
 import torch
 
+from oracle import reference_attend as R
 from tests import parity_util as U
 
 pytestmark = pytest.mark.gpu
@@ -20,7 +21,13 @@ CASES = [
     (1, 640, 2, 2, 128, 512, 32),     # default windows, D = 128
     (1, 1000, 2, 2, 64, 512, 32),     # ragged N with the default windows
     (1, 150, 2, 2, 128, 40, 5),       # odd number of offsets: the last offset pair of a step is half empty
-    (1, 260, 2, 1, 128, 70, 64),      # widest second window, D = 128 (fused four-wave backward kernels)
+    (1, 260, 2, 1, 128, 70, 64),      # second window of two offset blocks, D = 128
+    (1, 200, 2, 2, 64, 48, 65),       # second windows beyond 64 (the reference's backward stops at 32,
+    (1, 330, 2, 1, 128, 96, 100),     #   triton_two_simplicial_attention.py:586): offset rounds, offset blocks
+    (2, 160, 2, 2, 128, 160, 128),    # both windows >= N: full causal over three offset blocks
+    (1, 1, 1, 1, 128, 512, 32),       # a single row
+    (1, 17, 2, 1, 64, 512, 32),       # less than one tile
+    (2, 31, 4, 2, 128, 8, 32),        # less than one tile, second window wider than the sequence
 ]
 
 
@@ -37,24 +44,31 @@ def test_fwd_bwd_matches_oracle(b, n, hq, hk, d, w1, w2, unit_variance):
 def test_large_and_drifting_logits():
     """Logits that grow along the sequence by far more than 2^64 per window: exercises
     the paths of the forward that move the softmax reference point while accumulators
-    hold data.  q and k2 hold powers of two, so the bf16 operand q*k2 is exact and the
-    large logits carry no operand-rounding error (which would otherwise dominate any
-    comparison at this scale, for the reference's kernels as well)."""
+    hold data.  q and k2 hold powers of two and the softmax scale is chosen so that
+    scale * log2(e) = 2^-4, so the bf16 operand q * k2 * scale * log2(e) that the kernels feed
+    to the MFMA is exact and the large logits carry no operand-rounding error (which would
+    otherwise dominate any comparison at this scale, for the reference's kernels as well:
+    they round q * k1 * scale to bf16, triton_two_simplicial_attention.py:150-152, 182)."""
+    import math
+    from simplicial_attention_amd import SlidingTwoSimplicialAttention
     b, n, h, d, w1, w2 = 1, 256, 2, 128, 96, 16
+    scale = 2.0 ** -4 / math.log2(math.e)
     g = torch.Generator().manual_seed(21)
     q = torch.pow(2.0, torch.randint(-1, 2, (b, n, h, d), generator=g).float()).bfloat16()
     k2 = torch.pow(2.0, torch.randint(0, 2, (b, n, h, d), generator=g).float()).bfloat16()
     ramp = torch.linspace(0.2, 12.0, n).view(1, n, 1, 1)
-    k1 = (torch.randn(b, n, h, d, generator=g).abs() * ramp).bfloat16()
+    k1 = (torch.randn(b, n, h, d, generator=g).abs() * ramp * 2.0).bfloat16()
     v1, v2, dout = [torch.randn(b, n, h, d, generator=g).bfloat16() for _ in range(3)]
-    ins = (q, k1, k2, v1, v2, dout)
-    ref_out, ref_lse, ref_grads = U.oracle_fwd_bwd(*ins, w1, w2, dtype=torch.float64)
+    f64 = lambda t: t.double()
+    ref_out, ref_lse, ref_grads = R.windowed_banded_fwd_bwd(f64(q), f64(k1), f64(k2), f64(v1), f64(v2), f64(dout), w1, w2, scale=scale)
     assert float(ref_lse.max() - ref_lse.min()) > 100.0       # natural-log units
-    out, grads = U.hip_fwd_bwd(*ins, w1, w2)
+    ts = [t.cuda().requires_grad_(True) for t in (q, k1, k2, v1, v2)]
+    out = SlidingTwoSimplicialAttention.apply(*ts, w1, w2, True, scale)
+    grads = torch.autograd.grad(out, ts, dout.cuda())
     assert torch.isfinite(out.float()).all()
     row = U.compare('out', out, ref_out)
     assert row['bad'] == 0 and row['rel_fro'] <= 1e-2, row
-    # gradients reach magnitudes of 30-60 here (k1 is scaled up to 12x): relative check only
+    # gradients reach magnitudes of 30-60 here (k1 is scaled up to 24x): relative check only
     for name, got, ref in zip(U.NAMES[1:], grads, ref_grads):
         row = U.compare(name, got, ref)
         print('  ', row, flush=True)
