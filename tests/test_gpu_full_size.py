@@ -5,9 +5,13 @@ The CPU oracle cannot cover all (batch, head) slices of these shapes in test tim
     (forward and all five gradients, all 8192 rows), and the other slices through batch /
     head independence: permuting the slices of the inputs permutes the outputs bit for bit;
   * the layer shape of config 5 (grouped heads, dim_head 64) the same way;
-  * config 4 (N = 32768) is checked through translation equivariance of the windows: the
-    last rows of the full sequence must equal a run on the cropped sequence that still
-    holds every row those queries can reach.
+  * config 4 (N = 32768): one complete (batch, head) slice against the banded fp32 oracle
+    (all 32768 rows, forward and five gradients), and translation equivariance of the
+    windows: the last rows of the full sequence must equal a run on the cropped sequence
+    that still holds every row those queries can reach;
+  * config 1 exactly (the reference's CPU-runnable case: B=1, H=4, N=128, D=32, float32
+    N(0,1) inputs, full causal): the HIP path with both windows = N against autograd
+    through the dense naive attend.
 """
 import pytest
 import torch
@@ -97,3 +101,42 @@ def test_config4_translation_equivariance():
     assert rel(out[:, first:], out_c[:, off:]) <= 1e-2
     for a, c_ in zip(grads, grads_c):
         assert rel(a[:, first:], c_[:, off:]) <= 1e-2
+
+
+def test_config4_one_slice_against_oracle():
+    """One complete (batch, head) slice of config 4, all 32768 rows: output and the five
+    gradients against the banded fp32 CPU oracle (about 15 s of CPU time)."""
+    b, n, h, d, w1, w2 = 1, 32768, 16, 128, 512, 32
+    g = torch.Generator(device='cpu').manual_seed(3)
+    mk = lambda s: (torch.randn(b, n, h, d, generator=g) * s).bfloat16()
+    q, k1, k2, v1, v2 = (mk(d ** -0.5) for _ in range(5))
+    dout = mk(1.0)
+    out, grads = _run(*(t.cuda() for t in (q, k1, k2, v1, v2, dout)), w1, w2)
+    sh = 11
+    cut = lambda t: t[:, :, sh:sh + 1].contiguous()
+    ref_out, _, ref_grads = U.oracle_fwd_bwd(*(cut(t) for t in (q, k1, k2, v1, v2, dout)), w1, w2)
+    U.check_all(cut(out.cpu()), [cut(t.cpu()) for t in grads], ref_out, ref_grads)
+
+
+def test_config1_full_causal_against_dense_naive_attend():
+    """BASELINE config 1 on the HIP path: B=1, H=4, N=128, D=32, float32 N(0,1) inputs from a
+    fixed seed, full causal (both windows = N, the case of the reference's test_triton.py:65-80),
+    output and the autograd gradients of all five inputs against the dense naive attend
+    (simplicial_attention.py:78-127 restated in oracle/reference_attend.py, layout b h n d).
+    The kernels compute on bf16 operands: the oracle takes the bf16-rounded values, and the
+    reference's own tolerances for unit-variance inputs apply (tests/parity_util.py)."""
+    from oracle import reference_attend as R
+    from simplicial_attention_amd import sliding_two_simplicial_attn
+    b, h, n, d = 1, 4, 128, 32
+    g = torch.Generator(device='cpu').manual_seed(0)
+    q, k1, k2, v1, v2, dout = (torch.randn(b, h, n, d, generator=g) for _ in range(6))      # b h n d, float32
+    rounded = [t.bfloat16().float() for t in (q, k1, k2, v1, v2, dout)]
+    leaves = [t.clone().requires_grad_(True) for t in rounded[:5]]
+    ref_out = R.naive_two_simplicial_attend(leaves[0], (leaves[1], leaves[2]), (leaves[3], leaves[4]), causal=True)
+    ref_grads = torch.autograd.grad(ref_out, leaves, rounded[5])
+    to_kernel = lambda t: t.transpose(1, 2).contiguous()                                    # b n h d
+    ts = [to_kernel(t).cuda().requires_grad_(True) for t in (q, k1, k2, v1, v2)]
+    out = sliding_two_simplicial_attn(ts[0], (ts[1], ts[2]), (ts[3], ts[4]), w1=n, w2=n, causal=True)
+    assert out.dtype is torch.float32 and out.shape == (b, n, h, d)
+    grads = torch.autograd.grad(out, ts, to_kernel(dout).cuda())
+    U.check_all(out, grads, to_kernel(ref_out.detach()), [to_kernel(t) for t in ref_grads], unit_variance=True)

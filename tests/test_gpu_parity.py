@@ -177,3 +177,51 @@ def test_strided_views_need_no_copy():
     assert torch.equal(out_s, out_c)
     for x in range(5):
         assert torch.equal(gpk.view(b, n, h, 5, d)[:, :, :, x], grads_c[x])
+
+
+def test_each_backward_entry_point_against_the_oracle():
+    """sa2_bwd_delta, sa2_bwd_dq_dkv2 (with and without the forward's saved partials) and
+    sa2_bwd_dkv1 called one by one through the C ABI, each output against the CPU oracle."""
+    from simplicial_attention_amd import _native
+    lib = _native.load()
+    arg = _native.tensor_arg
+    b, n, hq, hk, d, w1, w2 = 2, 300, 4, 2, 128, 100, 40
+    ins = U.make_inputs(b, n, hq, hk, d, seed=77, std=d ** -0.5)
+    ref_out, ref_lse, ref_grads = U.oracle_fwd_bwd(*ins, w1, w2)
+    q, k1, k2, v1, v2, dout = (t.cuda() for t in ins)
+    prob = _native.problem(b, n, hq, hk, d, w1, w2, True, d ** -0.5)
+    sh = torch.cuda.current_stream().cuda_stream
+    out, res = torch.empty_like(q), torch.empty_like(q)
+    lse = torch.empty(b, hq, n, dtype=torch.float32, device='cuda')
+    t_save = torch.empty(lib.sa2_saved_t_bytes(prob), dtype=torch.uint8, device='cuda')
+    m_save = torch.empty(lib.sa2_saved_m_bytes(prob), dtype=torch.uint8, device='cuda')
+    saved = _native.saved_arg(t_save, m_save)
+    _native.check(lib.sa2_fwd(prob, arg(q), arg(k1), arg(k2), arg(v1), arg(v2), arg(out), arg(res), lse.data_ptr(), saved, sh))
+    # delta = sum_d out * dout
+    delta = torch.full_like(lse, float('nan'))
+    _native.check(lib.sa2_bwd_delta(prob, arg(out), arg(res), arg(dout), delta.data_ptr(), sh))
+    torch.cuda.synchronize()
+    want_delta = (ref_out * ins[5].float()).sum(-1).transpose(1, 2)                 # (b, h, n)
+    assert torch.allclose(delta.cpu(), want_delta, atol=2e-2, rtol=1e-2)
+    assert torch.allclose(lse.cpu(), ref_lse, atol=2e-2, rtol=1e-2)
+    ws_bytes = lib.sa2_bwd_workspace_bytes(prob)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device='cuda')
+    for use_saved in (True, False):
+        dq = torch.full_like(q, float('nan'))
+        dk2, dv2 = torch.full_like(k2, float('nan')), torch.full_like(v2, float('nan'))
+        _native.check(lib.sa2_bwd_dq_dkv2(prob, arg(q), arg(k1), arg(k2), arg(v1), arg(v2), arg(dout), lse.data_ptr(),
+                                          delta.data_ptr(), saved if use_saved else None, arg(dq), arg(dk2), arg(dv2),
+                                          ws.data_ptr(), ws_bytes, sh))
+        torch.cuda.synchronize()
+        for name, got, ref in (('dq', dq, ref_grads[0]), ('dk2', dk2, ref_grads[2]), ('dv2', dv2, ref_grads[4])):
+            row = U.compare(name, got, ref)
+            print('  ', use_saved, row, flush=True)
+            assert row['bad'] == 0 and row['rel_fro'] <= 1e-2, (use_saved, row)
+    dk1, dv1 = torch.full_like(k1, float('nan')), torch.full_like(v1, float('nan'))
+    _native.check(lib.sa2_bwd_dkv1(prob, arg(q), arg(k1), arg(k2), arg(v1), arg(v2), arg(dout), lse.data_ptr(), delta.data_ptr(),
+                                   arg(dk1), arg(dv1), sh))
+    torch.cuda.synchronize()
+    for name, got, ref in (('dk1', dk1, ref_grads[1]), ('dv1', dv1, ref_grads[3])):
+        row = U.compare(name, got, ref)
+        print('  ', row, flush=True)
+        assert row['bad'] == 0 and row['rel_fro'] <= 1e-2, row
