@@ -43,26 +43,156 @@ def attended_triples(n, w1, w2):
     return sum(min(i + 1, w1) * min(i + 1, w2) for i in range(n))
 
 
-def cpu_baseline(N, D, w1, w2, slices):
-    """The banded fp32 CPU oracle (a port of the reference algorithm; the reference
-    has no CPU implementation of the windowed path) on `slices` complete (batch, head)
-    slices of the workload, forward + backward, timed once."""
+def _median_time(fn, runs):
+    ts = []
+    for _ in range(runs):
+        t0 = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t0)
+    return statistics.median(ts), ts
+
+
+def cpu_baseline(N, D, w1, w2, slices, runs=3, naive_runs=5):
+    """Two CPU legs on the host cores, both the fp32 restatement of the reference algorithm
+    (`kind` "port": the reference's windowed path has no CPU implementation, its dense
+    `naive_two_simplicial_attend` is a dozen lines of PyTorch that the oracle restates):
+
+    `value`: the banded oracle, forward + backward, on `slices` complete (batch, head) slices
+             of the benchmarked workload; median of `runs` runs.
+    `naive_config1`: the dense naive attend at BASELINE config 1 (B=1, H=4, N=128, D=32, causal,
+             N(0,1) inputs), forward and forward + backward through autograd; median of
+             `naive_runs` runs each.  This is the reference's own CPU-runnable case.
+    """
     import torch
     from oracle import reference_attend as R
     g = torch.Generator().manual_seed(2)
     q, k1, k2, v1, v2 = [(torch.randn(1, N, slices, D, generator=g) * D ** -0.5).bfloat16().float() for _ in range(5)]
     dout = torch.randn(1, N, slices, D, generator=g).bfloat16().float()
-    t0 = time.perf_counter()
-    R.windowed_banded_fwd_bwd(q, k1, k2, v1, v2, dout, w1, w2, chunk=64)
-    t = time.perf_counter() - t0
+    t, ts = _median_time(lambda: R.windowed_banded_fwd_bwd(q, k1, k2, v1, v2, dout, w1, w2, chunk=64), runs)
     flops = 18 * D * slices * attended_triples(N, w1, w2)
+
+    # config 1: dense, causal over both key axes: sum_i (i+1)^2 attended triples per (batch, head)
+    b1, h1, n1, d1 = 1, 4, 128, 32
+    g = torch.Generator().manual_seed(1)
+    x = [torch.randn(b1, h1, n1, d1, generator=g).requires_grad_(True) for _ in range(5)]
+    do1 = torch.randn(b1, h1, n1, d1, generator=g)
+    trip1 = sum((i + 1) ** 2 for i in range(n1))
+
+    def naive_fwd():
+        with torch.no_grad():
+            R.naive_two_simplicial_attend(x[0], (x[1], x[2]), (x[3], x[4]), causal=True)
+
+    def naive_fwd_bwd():
+        o = R.naive_two_simplicial_attend(x[0], (x[1], x[2]), (x[3], x[4]), causal=True)
+        torch.autograd.grad(o, x, do1)
+    naive_fwd_bwd()
+    tf, tfs = _median_time(naive_fwd, naive_runs)
+    tb, tbs = _median_time(naive_fwd_bwd, naive_runs)
     return {
         'value': round(flops / t / 1e12, 4), 'unit': 'TFLOP/s', 'cores': torch.get_num_threads(), 'kind': 'port',
         'tokens_per_s': round(N * slices / t, 1),
         'sample': f'{slices} of the workload\'s (batch, head) slices, all {N} rows each, D={D} w1={w1} w2={w2}, '
-                  f'fp32 banded oracle fwd+bwd, one run of {t:.1f} s; tokens_per_s counts rows of these slices; '
-                  f'host cpu_count={os.cpu_count()}',
+                  f'fp32 banded oracle fwd+bwd, median of {runs} runs ({", ".join("%.1f" % v for v in ts)} s); '
+                  f'tokens_per_s counts rows of these slices; host cpu_count={os.cpu_count()}',
+        'naive_config1': {
+            'workload': 'cfg1_naive_b1_h4_n128_d32_causal_fp32',
+            'fwd_ms': round(tf * 1e3, 3), 'fwd_bwd_ms': round(tb * 1e3, 3),
+            'fwd_tokens_per_s': round(b1 * n1 / tf, 1), 'fwd_bwd_tokens_per_s': round(b1 * n1 / tb, 1),
+            'fwd_gflops': round(4 * d1 * b1 * h1 * trip1 / tf / 1e9, 2),
+            'fwd_bwd_gflops': round(18 * d1 * b1 * h1 * trip1 / tb / 1e9, 2),
+            'runs': naive_runs,
+            'note': 'dense naive attend (what the reference tests against), autograd backward; flop counted over the '
+                    'causally attended triples only, as for the GPU figures',
+        },
     }
+
+
+def source_digest():
+    """sha256 over the kernel sources: ties a stored counter measurement to the code it was taken on."""
+    import glob
+    import hashlib
+    h = hashlib.sha256()
+    csrc = os.path.join(ROOT, 'simplicial_attention_amd', 'csrc')
+    for f in sorted(glob.glob(os.path.join(csrc, '*.hpp')) + glob.glob(os.path.join(csrc, '*.hip'))):
+        h.update(os.path.basename(f).encode())
+        h.update(open(f, 'rb').read())
+    return h.hexdigest()[:16]
+
+
+TRAFFIC_FILE = os.path.join(ROOT, 'profiles', 'hbm_traffic.json')
+# the one MFMA kernel behind each single-kernel bench entry (substring of the kernel symbol)
+ENTRY_KERNEL = {'fwd': 'fwd', 'bwd_dq_dk2_pass': 'bwd_q_kernel', 'bwd_dkv1': 'bwd_kv8_kernel'}
+
+
+def kernel_symbol(entry, D, w2):
+    if entry == 'fwd':
+        return 'sa2::fwd8_kernel<64, 32>' if (D == 64 and w2 <= 32) else 'sa2::fwd_kernel<%d>' % D
+    if entry == 'bwd_dq_dk2_pass':
+        return 'sa2::bwd_q_kernel<%d, true>' % D
+    if entry == 'bwd_dkv1':
+        return 'sa2::bwd_kv8_kernel<%d, %d>' % (D, 3 if D == 128 else 2)
+    return None
+
+
+def stored_traffic(workload, entry):
+    """HBM bytes per launch of `entry` at `workload`, from the tracked counter summary (written by
+    `--traffic-from`); None with a note if there is none or it was taken on other kernel sources."""
+    try:
+        rec = json.load(open(TRAFFIC_FILE))
+    except (OSError, ValueError):
+        return None, 'no profiles/hbm_traffic.json'
+    e = rec.get('workloads', {}).get(workload, {}).get(entry)
+    if e is None:
+        return None, 'no counter run stored for this entry and workload'
+    if rec.get('source_digest') != source_digest():
+        return None, 'stored counter run (%s bytes) was taken on other kernel sources: rerun the --pmc passes' % e['total_bytes']
+    return e['total_bytes'], 'rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE, scaled by a 1 GiB copy; profiles/hbm_traffic.json'
+
+
+def traffic_from(directory):
+    """Reads the counter CSVs of the rocprofv3 --pmc passes under `directory` (sub-directories
+    <entry>_FETCH_SIZE, <entry>_WRITE_SIZE for entry in copy and the kernels; each pass is
+    `rocprofv3 --pmc <counter> -d <directory>/<entry>_<counter> -o out --output-format csv --
+    python3 bench.py --only <entry> [--workload W] --kernel-iters 2 --cpu-slices 0`) and writes
+    profiles/hbm_traffic.json."""
+    import csv
+    import glob
+
+    def per_dispatch(sub, counter, kernel_part):
+        vals = []
+        for f in glob.glob(os.path.join(directory, sub, '**', '*counter_collection.csv'), recursive=True):
+            for row in csv.DictReader(open(f)):
+                name = row.get('Kernel_Name', '')
+                if kernel_part == 'fwd' and not ('fwd_kernel' in name or 'fwd8_kernel' in name):
+                    continue
+                if row.get('Counter_Name') == counter and kernel_part in name:
+                    vals.append(float(row['Counter_Value']))
+        return statistics.mean(vals) if vals else None
+    cf = per_dispatch('copy_FETCH_SIZE', 'FETCH_SIZE', 'copyBuffer')
+    cw = per_dispatch('copy_WRITE_SIZE', 'WRITE_SIZE', 'copyBuffer')
+    if not cf or not cw:
+        sys.exit('traffic_from: the copy calibration passes are missing under ' + directory)
+    kib = float(1 << 20)                     # the copy moves 1 GiB each way
+    f_fetch, f_write = kib / cf, kib / cw
+    rec = {'source_digest': source_digest(), 'calibration': {'copy_FETCH_SIZE': cf, 'copy_WRITE_SIZE': cw,
+                                                             'fetch_factor': round(f_fetch, 4), 'write_factor': round(f_write, 4)},
+           'workloads': {}}
+    for sub in sorted(os.listdir(directory)):
+        if not sub.endswith('_FETCH_SIZE') or sub.startswith('copy_'):
+            continue
+        tag = sub[:-len('_FETCH_SIZE')]                  # <workload>__<entry>
+        workload, entry = tag.split('__')
+        kern = ENTRY_KERNEL.get(entry)
+        if kern is None:
+            continue
+        fs = per_dispatch(sub, 'FETCH_SIZE', kern)
+        wsz = per_dispatch(tag + '_WRITE_SIZE', 'WRITE_SIZE', kern)
+        if fs is None or wsz is None:
+            continue
+        rd, wr = fs * f_fetch * 1024, wsz * f_write * 1024
+        rec['workloads'].setdefault(workload, {})[entry] = {'read_bytes': int(rd), 'written_bytes': int(wr), 'total_bytes': int(rd + wr)}
+    json.dump(rec, open(TRAFFIC_FILE, 'w'), indent=1, sort_keys=True)
+    print(json.dumps(rec))
 
 
 def main():
@@ -73,8 +203,12 @@ def main():
     ap.add_argument('--workload', default='cfg3_raw_kernel_b4_h8_n8192_d128_w512_w32', choices=sorted(WORKLOADS))
     ap.add_argument('--cpu-slices', type=int, default=4, help='(batch, head) slices of the CPU baseline sample (0 = skip)')
     ap.add_argument('--kernel-iters', type=int, default=5, help='launches per kernel for the per-kernel timing')
+    ap.add_argument('--traffic-from', default=None, metavar='DIR', help='no GPU work: read the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE passes under DIR and write profiles/hbm_traffic.json')
     ap.add_argument('--only', default=None, help='time only this entry through the C ABI (fwd, bwd_delta, bwd_dq_dkv2, bwd_dkv1, bwd_dq_dk2_pass), `copy`: a 1 GiB device copy that calibrates HBM counters; `module_cfg2`: the module forward of config 2 and the fused qkv-norm kernel; `train_cfg5`: one training step of the config-5 language model; for profiling')
     args = ap.parse_args()
+    if args.traffic_from:
+        traffic_from(args.traffic_from)
+        return
     if args.gpus != 1:
         print('bench.py: this build runs on one GPU; --gpus must be 1 (no multi-GPU path exists)', file=sys.stderr)
         sys.exit(2)
@@ -236,7 +370,7 @@ def main():
     # the forward's per-offset value partials, as the autograd Function keeps them
     saved = t_save = m_save = None
     from simplicial_attention_amd.two_simplicial_attention import save_partials_max_bytes
-    if w2 <= 32 and lib.sa2_saved_t_bytes(prob) <= save_partials_max_bytes():
+    if lib.sa2_saved_t_bytes(prob) <= save_partials_max_bytes():
         t_save = torch.empty(lib.sa2_saved_t_bytes(prob), dtype=torch.uint8, device=dev)
         m_save = torch.empty(lib.sa2_saved_m_bytes(prob), dtype=torch.uint8, device=dev)
         saved = _native.saved_arg(t_save, m_save)
@@ -247,21 +381,18 @@ def main():
                                                       arg(dv2), ws.data_ptr(), ws_bytes, sh)),
         'bwd_dkv1': (4, lambda: lib.sa2_bwd_dkv1(prob, *five, arg(dout), lse.data_ptr(), delta.data_ptr(), arg(dk1), arg(dv1), sh)),
     }
-    if w2 <= 32:
-        # the two-pass backward entry points, one pass (= one kernel) at a time
-        # the MFMA kernel of the dQ/dK2/dV2 entry point alone: the profiling build of the library
-        # launches only that kernel when SA2_BWD_PASS=first is set (the product library has no such switch)
-        plib = _native.load_profiling()
+    # the MFMA kernel of the dQ/dK2/dV2 entry point alone: the profiling build of the library launches only
+    # that kernel when SA2_BWD_PASS=first is set (the product library has no such switch)
+    plib = _native.load_profiling()
 
-        def dq_dk2_kernel_alone():
-            os.environ['SA2_BWD_PASS'] = 'first'
-            try:
-                return plib.sa2_bwd_dq_dkv2(prob, *five, arg(dout), lse.data_ptr(), delta.data_ptr(), saved, arg(dq),
-                                            arg(dk2), arg(dv2), ws.data_ptr(), ws_bytes, sh)
-            finally:
-                del os.environ['SA2_BWD_PASS']
-        launches['bwd_dq_dk2_pass'] = (3, dq_dk2_kernel_alone)
-        # bwd_dkv1 is a single launch (one kernel produces dK1 and dV1)
+    def dq_dk2_kernel_alone():
+        os.environ['SA2_BWD_PASS'] = 'first'
+        try:
+            return plib.sa2_bwd_dq_dkv2(prob, *five, arg(dout), lse.data_ptr(), delta.data_ptr(), saved, arg(dq),
+                                        arg(dk2), arg(dv2), ws.data_ptr(), ws_bytes, sh)
+        finally:
+            del os.environ['SA2_BWD_PASS']
+    launches['bwd_dq_dk2_pass'] = (3, dq_dk2_kernel_alone)
     kernels = {}
     if args.only is not None:
         # the later kernels read what the earlier ones wrote: run the chain once, untimed
@@ -288,23 +419,15 @@ def main():
         print(json.dumps({'workload': args.workload, 'kernels': kernels}))
         return
     hbm_bytes = {'fwd': 7 * B * N * H * D * 2 + 4 * B * H * N, 'bwd_delta': 3 * B * N * H * D * 2 + 4 * B * H * N}
-    # entries that are exactly one kernel launch (the two-pass entry points are timed per pass)
-    multi = () if w2 > 32 else ('bwd_dq_dkv2',)
+    # entries that are exactly one kernel launch (the dQ/dK2/dV2 entry point launches several: its MFMA kernel is
+    # timed alone as bwd_dq_dk2_pass)
+    multi = ('bwd_dq_dkv2',)
     single = [k for k in kernels if kernels[k]['contractions'] and k not in multi]
     dom = max(single, key=lambda k: kernels[k]['ms'])
     achieved = kernels[dom]['tflops']
-    symbols = {'fwd': 'sa2::fwd8_kernel<%d, %d>' % (D, 32 if w2 <= 32 else 64), 'bwd_dq_dk2_pass': 'sa2::bwd_q8_kernel<%d, true>' % D}
-    if w2 <= 32:
-        symbols['bwd_dkv1'] = 'sa2::bwd_kv8_kernel<%d, %d>' % (D, 3 if D == 128 else 2)
-    # HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of `--only <entry>` on this
-    # workload, scaled by what the same counters read for a 1 GiB device copy (profiles/pmc_cfg3_mfma_kernels.txt)
-    measured_traffic = {
-        'cfg3_raw_kernel_b4_h8_n8192_d128_w512_w32': {
-            'fwd': 2682106604, 'bwd_dq_dk2_pass': 736942192, 'bwd_dkv1': 710897605},
-    }
-    traffic = measured_traffic.get(args.workload, {}).get(dom)
-    roofline = {'bound': 'mfma', 'kernel': dom, 'kernel_symbol': symbols.get(dom), 'achieved': achieved, 'peak': PEAK_BF16_TFLOPS, 'unit': 'TFLOP/s',
-                'frac': round(achieved / PEAK_BF16_TFLOPS, 4), 'traffic': traffic,
+    traffic, traffic_note = stored_traffic(args.workload, dom)
+    roofline = {'bound': 'mfma', 'kernel': dom, 'kernel_symbol': kernel_symbol(dom, D, w2), 'achieved': achieved, 'peak': PEAK_BF16_TFLOPS, 'unit': 'TFLOP/s',
+                'frac': round(achieved / PEAK_BF16_TFLOPS, 4), 'traffic': traffic, 'traffic_note': traffic_note,
                 'launch_ms': kernels[dom]['ms'],
                 'flops_per_launch': kernels[dom]['contractions'] * unit}
 
