@@ -40,12 +40,19 @@ template <int D>
 struct FwdCfg {
     static constexpr int KS = D / 16;
     static constexpr int DT = D / 32;
-    static constexpr int PITCH = tile_pitch<D>();
-    static constexpr int TILE = 32 * PITCH;           // K1 tile, read row-major
-    static constexpr int VPITCH = tr_pitch<D>();
-    static constexpr int VTILE = 32 * VPITCH;         // V1 tile, read through transposed reads only
-    static constexpr int BUF = TILE + VTILE;          // one ring buffer: a K1 tile and a V1 tile
-    static constexpr int NBUF = 3;
+    static constexpr int PITCH = tile_pitch<D>();     // staged q / k2 / v2 rows
+    static constexpr int TILE = 32 * PITCH;
+    // K1 / V1 ring tiles are written by direct-to-LDS loads: one wave instruction moves 64 pieces of 16 bytes to
+    // 1 KiB of consecutive LDS, a "chunk" of RPC rows.  Inside a chunk the 64-byte segments of the rows are
+    // interleaved, [segment][row][64 bytes], and chunks start 1040 bytes apart: the 16 rows that a quarter of a
+    // row-fragment read touches, and the 4 rows x 64 bytes of a transposed read, then cover all 64 banks.
+    static constexpr int NSEG = D * 2 / 64;           // 64-byte segments per row
+    static constexpr int RPC = 16 / NSEG;             // rows per chunk
+    static constexpr int NCH = 32 / RPC;              // chunks per tile
+    static constexpr int CP = 1040;                   // chunk pitch
+    static constexpr int DTILE = NCH * CP;
+    static constexpr int BUF = 2 * DTILE;             // one ring buffer: a K1 tile and a V1 tile
+    static constexpr int NBUF = 4;
     static constexpr int RING = NBUF * BUF;
     static constexpr int APITCH = D + 4;              // floats per row of the shared accumulator
     static constexpr int ACC = 32 * APITCH * 4;
@@ -57,9 +64,26 @@ struct FwdCfg {
     static constexpr int MASKS = V2S + KSLOTS * PITCH; // additive masks (0 / -inf) of the diagonal tile and of up to two lower-edge tiles
     static constexpr int MASK = 16 * 64 * 4;          // one table: [4 quarters][64 lanes][4 floats]
     static constexpr int LDS = MASKS + 3 * MASK;
+    // byte offset of element (row, d) inside a ring tile
+    static constexpr int ring_off(int row, int d) {
+        return (row / RPC) * CP + (d / 32) * (RPC * 64) + (row % RPC) * 64 + (d % 32) * 2;
+    }
+    static_assert(RING - CP < 65536, "the LDS address of a direct load travels in 16 bits of M0");
     static constexpr int PPR = D / 8;                 // 16-byte pieces per row
     static constexpr int PIECES = 32 * PPR;           // ... per tile
 };
+
+// One direct-to-LDS load: lane l of the wave fetches the 16 bytes at base + offset_l and they land at LDS address
+// lds_addr + 16 l (both base and lds_addr are wave-uniform).  Counted by vmcnt like any global load; written as
+// assembly so that the compiler does not order the kernel's ordinary LDS reads behind it - the kernel waits for
+// the transfer itself (wait_loads) before the barrier that publishes the tile.
+__device__ __forceinline__ void load_to_lds16(const char *base, uint32_t lane_offset, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_offset), "s"(base), "s"(lds_addr) : "memory");   // (m0 is reserved: the compiler keeps nothing in it across statements)
+}
+template <int N_LEFT>
+__device__ __forceinline__ void wait_loads() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N_LEFT) : "memory");
+}
 
 template <int D>
 __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
@@ -100,37 +124,34 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
     const int U = R * NT;
     auto tile_of = [&](int n) { return n == 0 ? t_hi : t_lo + n - 1; };
 
-    // ---- ring staging: the first PIECES threads move one 16-byte piece of K1 and of V1 per tile
-    const bool stager = tid < C::PIECES;
-    const int st_row = tid / PPR, st_col = (tid % PPR) * 16;
-    const int st_off = st_row * PITCH + st_col;
-    const int st_off_v = C::TILE + st_row * C::VPITCH + st_col;
-    u32x4 st_k = {0u, 0u, 0u, 0u}, st_v = {0u, 0u, 0u, 0u};
-    int n_load = 0, u_load = 0;                       // sequence index (within the round) / running count of the next load
-    // address = tile base (uniform, on the scalar unit) + this thread's row and column (32 bits); only
+    // ---- ring staging: direct-to-LDS loads, wave w moves chunk(s) w of the K1 tile and of the V1 tile.  Lane p of a
+    // chunk load fetches row (p / 4) % RPC, segment p / (4 RPC), piece p % 4 of the segment
+    const bool stager = wave < C::NCH;                           // D = 64: four chunks per tile, waves 0-3 stage
+    const int st_row = (wave % C::NCH) * C::RPC + (lane >> 2) % C::RPC;
+    const int st_col = (lane / (4 * C::RPC)) * 64 + (lane & 3) * 16;
+    int n_load = 0;                                   // sequence index (within the round) of the next load
+    int b_load = 0;                                   // ring buffer of the next load
+    // address = tile base (uniform, on the scalar unit) + this lane's row and column (32 bits); only
     // the diagonal tile can reach past the last row, so only it needs a clamped row
     const int st_row_diag = i0 + st_row < N ? st_row : N - 1 - i0;
     const uint32_t so_k = (uint32_t)(st_row * (int)p.k1.sn + st_col), so_v = (uint32_t)(st_row * (int)p.v1.sn + st_col);
     const uint32_t so_k_diag = (uint32_t)(st_row_diag * (int)p.k1.sn + st_col), so_v_diag = (uint32_t)(st_row_diag * (int)p.v1.sn + st_col);
+    const uint32_t lds_chunk = (uint32_t)(uintptr_t)lds + (wave % C::NCH) * C::CP;
     auto issue_loads = [&]() {
         const int t = tile_of(n_load);
         const char *kb = k1g + (int64_t)(32 * t) * p.k1.sn;
         const char *vb = v1g + (int64_t)(32 * t) * p.v1.sn;
         if (stager) {
-            st_k = ld_global16(kb + (n_load == 0 ? so_k_diag : so_k));
-            st_v = ld_global16(vb + (n_load == 0 ? so_v_diag : so_v));
+            load_to_lds16(kb, n_load == 0 ? so_k_diag : so_k, lds_chunk + b_load);
+            load_to_lds16(vb, n_load == 0 ? so_v_diag : so_v, lds_chunk + b_load + C::DTILE);
         }
-        ++u_load;
         n_load = (n_load == NT - 1) ? 0 : n_load + 1;
+        b_load = (b_load == (C::NBUF - 1) * C::BUF) ? 0 : b_load + C::BUF;
     };
-    auto write_stage = [&](int buf_off) {
-        if (stager) {
-            *reinterpret_cast<u32x4 *>(lds + buf_off + st_off) = st_k;
-            *reinterpret_cast<u32x4 *>(lds + buf_off + st_off_v) = st_v;
-        }
-    };
-    const int k_lane = c * PITCH + 16 * hf;          // K1 fragment: row c, pieces 2*kk + hf
-    const int v_lane = C::TILE + tr_lane_off<D, C::VPITCH>(lane);
+    // K1 fragment kk of row c: segment kk / 2, pieces 2 (kk % 2) + hf
+    const int k_lane = (c / C::RPC) * C::CP + (c % C::RPC) * 64 + 16 * hf;
+    // V1 transposed read: the lane's 8 bytes of row 4 hf + (lane % 16) / 4, d = 16 (lane & 1) + 8 (lane / 16 % 2) + 4 (lane % 4 / 2)
+    const int v_lane = C::DTILE + C::ring_off(4 * hf + ((lane & 15) >> 2), 16 * (lane & 1) + 8 * ((lane >> 4) & 1) + 4 * ((lane & 3) >> 1));
 
     // ---- shared output accumulator and exchange areas
     float *acc_sh = reinterpret_cast<float *>(lds + C::RING);              // [32][APITCH]
@@ -195,32 +216,31 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
     bool fresh = true;         // the row has not met an attended entry yet
     float l = 0.f;             // this lane's part of the row sum, relative to M
 
-    // ring protocol: step u lives in buffer u % 3; it is written at the end of step u - 2 from
-    // registers loaded at the end of step u - 3 and read (as fragments) from step u - 1 on
-    int b_cur = 0, b_nxt = C::BUF, b_nn = 2 * C::BUF;
+    // ring protocol: step u lives in buffer u % 4.  Its transfer starts behind the barrier of step u - 3 (every wave
+    // has then finished step u - 4, the last reader of that buffer) and must have landed before the barrier of step
+    // u - 1, in which its K1 fragments are read: two steps of time for the memory latency.
+    int b_cur = 0, b_nxt = C::BUF;
     issue_loads();
-    write_stage(0);
-    if (U > 1) {
-        issue_loads();
-        write_stage(C::BUF);
-    }
+    if (U > 1) issue_loads();
     if (U > 2) issue_loads();
     int u = 0;
-
-    // end of a step: the tile two steps ahead goes to its buffer, the next global loads start
-    auto stage_ahead = [&]() {
-        if (u + 2 < U) {
-            write_stage(b_nn);
-            if (u_load < U) issue_loads();
+    wait_loads<0>();
+    // start of step u: the tile of step u + 1 has landed (at most the transfers of step u + 2 are still in flight),
+    // everything is published, the transfer of step u + 3 starts
+    auto open_step = [&]() {
+        if (stager) {
+            if (u + 2 < U) wait_loads<2>();
+            else wait_loads<0>();
         }
-        const int t = b_cur;
+        __syncthreads();
+        if (u + 3 < U) issue_loads();
+    };
+    auto close_step = [&]() {
         b_cur = b_nxt;
-        b_nxt = b_nn;
-        b_nn = t;
+        b_nxt = (b_nxt == (C::NBUF - 1) * C::BUF) ? 0 : b_nxt + C::BUF;
         ++u;
     };
-
-    __syncthreads();           // staged rows, the zeroed accumulator and the first two tiles are visible
+    __syncthreads();           // the staged rows, the mask tables and the zeroed accumulator are visible
 
     for (int r = 0; r < R; ++r) {
         const int dlt = 8 * r + wave;
@@ -265,14 +285,14 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
             for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
                 for (int k2s = 0; k2s < 2; ++k2s) {
-                    vf[dt][k2s][0] = lds_read_tr<D, C::VPITCH>(vbase, 16 * k2s, 32 * dt);
-                    vf[dt][k2s][1] = lds_read_tr<D, C::VPITCH>(vbase, 16 * k2s + 8, 32 * dt);
+                    vf[dt][k2s][0] = lds_read_tr<D, 0>(vbase + C::ring_off(16 * k2s, 32 * dt), 0, 0);
+                    vf[dt][k2s][1] = lds_read_tr<D, 0>(vbase + C::ring_off(16 * k2s + 8, 32 * dt), 0, 0);
                 }
         };
         auto load_kf = [&](int buf_off) {
             const char *kbase = lds + buf_off + k_lane;
 #pragma unroll
-            for (int kk = 0; kk < KS; ++kk) kf[kk] = ld_lds16(kbase + 32 * kk);
+            for (int kk = 0; kk < KS; ++kk) kf[kk] = ld_lds16(kbase + (kk >> 1) * (C::RPC * 64) + (kk & 1) * 32);
         };
         auto value_products = [&](const u32x4 (&pb)[2], bool next_kf) {
             if (next_kf) load_kf(b_nxt);
@@ -316,15 +336,15 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
             // (a wave that is off stays off: later rounds only have larger offsets, so its fragment
             // registers need not follow the ring)
             for (int n = 0; n < NT; ++n) {
-                __syncthreads();
-                stage_ahead();
+                open_step();
+                close_step();
             }
         } else {
             int n = 0;
             if (r == 0) {
                 // ---- the wave's very first step, the diagonal tile of its first offset: every valid row
                 // attends an entry of it, so this is where the rows get their softmax reference M
-                __syncthreads();
+                open_step();
                 f32x16 X = zero16();
                 logit_chain(X);
                 {
@@ -347,7 +367,7 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
                 u32x4 pb[2];
                 exponentials(X, pb);
                 value_products(pb, 1 < NT);
-                stage_ahead();
+                close_step();
                 n = 1;
             }
             // ---- all other steps.  The logit chain starts from -M (from -inf in lanes without a valid
@@ -355,17 +375,10 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
             // tiles that the window's lower edge crosses, so its result is the exponent and no mask or
             // subtraction code follows it.  A row's reference moves only if its row sum says that weights
             // outgrew the safe range.
-            // The two waves of a SIMD advance in step (their dependent MFMA chains interleave one
-            // instruction at a time), so with the barrier at the same place both would run their
-            // exponentials at the same time and leave the MFMA pipe idle.  The second wave of each SIMD
-            // (waves 4-7) therefore takes the step's barrier after its logit chain instead of before it:
-            // behind every barrier the first group starts a logit chain while the second group starts its
-            // exponentials.  Reading tile n before the step's barrier is safe: the barrier before published it.
-            const bool late = wave >= 4;
             float nm = col_ok ? -M : -INFINITY;
             u32x4 pb[2];
             for (; n < NT; ++n) {
-                if (!late) __syncthreads();
+                open_step();
                 f32x16 X;
                 if (n < n_masked) {
                     const char *mk = lds + C::MASKS + n * C::MASK + lane * 16;
@@ -382,7 +395,6 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
                     for (int rr = 0; rr < 16; ++rr) X[rr] = nm;
                 }
                 logit_chain(X);
-                if (late) __syncthreads();
                 const float l_before = l;
                 exponentials(X, pb);
                 if (wave_any(!(l < kBig))) {
@@ -401,7 +413,7 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
                     exponentials(X, pb);
                 }
                 value_products(pb, n + 1 < NT);
-                stage_ahead();
+                close_step();
             }
         }
 
