@@ -80,6 +80,18 @@ struct FwdCfg {
 __device__ __forceinline__ void load_to_lds16(const char *base, uint32_t lane_offset, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_offset), "s"(base), "s"(lds_addr) : "memory");   // (m0 is reserved: the compiler keeps nothing in it across statements)
 }
+// sixteen registers holding x (each element is pinned to a register of its own: left to itself the compiler
+// copies a whole undefined tuple first and then overwrites fifteen of its registers)
+__device__ __forceinline__ f32x16 splat16(float x) {
+    f32x16 r;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        float t = x;
+        asm("" : "+v"(t));
+        r[e] = t;
+    }
+    return r;
+}
 template <int N_LEFT>
 __device__ __forceinline__ void wait_loads() {
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N_LEFT) : "memory");
@@ -268,14 +280,14 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
             // (the row sum takes the unrounded weights: v_dot2c_f32_bf16 on the packed pairs would be exact
             // for what the MFMA consumes, but dot instructions share the MFMA pipe and stall the other
             // wave's chains; the two sums differ by the mean of bf16 rounding errors, far below bf16 eps)
-            float ls = 0.f;
+            float ls = l;
 #pragma unroll
             for (int rr = 0; rr < 16; rr += 2) {
                 const float e0 = fast_exp2(X[rr]), e1 = fast_exp2(X[rr + 1]);
                 ls += e0 + e1;
                 pb[rr >> 3][(rr & 7) >> 1] = pack_bf16(e0, e1);
             }
-            l += ls;
+            l = ls;
         };
         // fragment reads of a step: the V1 fragments of the tile behind its logit chain, the K1 fragments of
         // the next tile in front of the value chain (they arrive behind it and the barrier)
@@ -294,21 +306,31 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
 #pragma unroll
             for (int kk = 0; kk < KS; ++kk) kf[kk] = ld_lds16(kbase + (kk >> 1) * (C::RPC * 64) + (kk & 1) * 32);
         };
+        // The fragment reads of a step sit between its MFMAs, a scheduling fence behind every MFMA and its reads
+        // keeps them there: the V1 fragments of the tile along its logit chain, the K1 fragments of the next tile
+        // along the value chain.
         auto value_products = [&](const u32x4 (&pb)[2], bool next_kf) {
-            if (next_kf) load_kf(b_nxt);
+            const char *kbase = lds + b_nxt + k_lane;
 #pragma unroll
-            for (int k2s = 0; k2s < 2; ++k2s)
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt) {
-                    u32x4 v = {vf[dt][k2s][0][0], vf[dt][k2s][0][1], vf[dt][k2s][1][0], vf[dt][k2s][1][1]};
-                    T[dt] = mfma32(v, pb[k2s], T[dt]);
-                }
+            for (int m = 0; m < 2 * DT; ++m) {
+                const int k2s = m / DT, dt = m % DT;
+                u32x4 v = {vf[dt][k2s][0][0], vf[dt][k2s][0][1], vf[dt][k2s][1][0], vf[dt][k2s][1][1]};
+                T[dt] = mfma32(v, pb[k2s], T[dt]);
+                if (next_kf) kf[m] = ld_lds16(kbase + (m >> 1) * (C::RPC * 64) + (m & 1) * 32);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         };
-        // S^T = K1 A^T on top of X
         auto logit_chain = [&](f32x16 &X) {
+            const char *vbase = lds + b_cur + v_lane;
+            __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int kk = 0; kk < KS; ++kk) X = mfma32(kf[kk], A[kk], X);
-            load_vf();
+            for (int kk = 0; kk < KS; ++kk) {
+                X = mfma32(kf[kk], A[kk], X);
+                const int k2s = kk / DT, dt = kk % DT;
+                vf[dt][k2s][0] = lds_read_tr<D, 0>(vbase + C::ring_off(16 * k2s, 32 * dt), 0, 0);
+                vf[dt][k2s][1] = lds_read_tr<D, 0>(vbase + C::ring_off(16 * k2s + 8, 32 * dt), 0, 0);
+                __builtin_amdgcn_sched_barrier(0);
+            }
         };
         // moves the reference of this lane's row up by `shift` (log2 units): what T and l hold is rescaled
         // (alpha = 2^-shift, or 1 for a row that holds nothing yet)
@@ -379,25 +401,22 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
             u32x4 pb[2];
             for (; n < NT; ++n) {
                 open_step();
-                f32x16 X;
+                f32x16 X = splat16(nm);
                 if (n < n_masked) {
                     const char *mk = lds + C::MASKS + n * C::MASK + lane * 16;
 #pragma unroll
                     for (int qq = 0; qq < 4; ++qq) {
                         const float4 m4 = *reinterpret_cast<const float4 *>(mk + qq * 1024);
-                        X[4 * qq] = m4.x + nm;
-                        X[4 * qq + 1] = m4.y + nm;
-                        X[4 * qq + 2] = m4.z + nm;
-                        X[4 * qq + 3] = m4.w + nm;
+                        X[4 * qq] += m4.x;
+                        X[4 * qq + 1] += m4.y;
+                        X[4 * qq + 2] += m4.z;
+                        X[4 * qq + 3] += m4.w;
                     }
-                } else {
-#pragma unroll
-                    for (int rr = 0; rr < 16; ++rr) X[rr] = nm;
                 }
                 logit_chain(X);
                 const float l_before = l;
                 exponentials(X, pb);
-                if (wave_any(!(l < kBig))) {
+                if (__builtin_expect(wave_any(!(l < kBig)), 0)) {
                     // rare: some row's weights outgrew the safe range; move its reference and redo the tile's weights
                     const float tmax = row_max(X);
                     auto sw = __builtin_amdgcn_permlane32_swap(as_u32(l), as_u32(l), false, false);
