@@ -36,14 +36,12 @@ template <int D, bool DQ>
 struct QCfg {
     static constexpr int KS = D / 16;
     static constexpr int DT = D / 32;
-    static constexpr int PITCH = tile_pitch<D>();
-    static constexpr int TILE = 32 * PITCH;           // a tile read row-major
-    static constexpr int TPITCH = tr_pitch<D>();
-    static constexpr int TRT = 32 * TPITCH;           // a tile read through transposed reads
-    // ring buffer: DQ: [K1, read both ways: swizzled layout of sa2_lds.hpp][V1 row-major];  DV: [K1 row-major][V1 transposed-read]
-    static constexpr int OFF_TR = DQ ? 0 : TILE;      // the tile read through transposed reads
-    static constexpr int OFF_V = TRT;                 // DQ only
-    static constexpr int BUF = TILE + TRT;
+    static constexpr int PITCH = tile_pitch<D>();     // staged q / do / k2 / v2 rows
+    static constexpr int TILE = 32 * PITCH;
+    // ring buffer: a K1 tile and a V1 tile, written by direct-to-LDS loads (layout: DmaTile; DQ reads K1 both ways)
+    using RT = DmaTile<D>;
+    static constexpr int OFF_V = RT::BYTES;
+    static constexpr int BUF = 2 * RT::BYTES;
     static constexpr int RING = 2 * BUF;
     static constexpr int SPITCH = D + 4;              // floats per row of the fp32 rows
     static constexpr int DQS = RING;                  // dq rows [32][SPITCH]            (DQ only)
@@ -129,38 +127,32 @@ __global__ __launch_bounds__(512) void bwd_q_kernel(KParams p, float *ws, int ha
     const int R = (nd + 7) / 8;
     const int U = R * NT;
 
-    // ---- ring staging: the first PIECES threads move one 16-byte piece of K1 and of V1 per tile
-    const bool stager = tid < C::PIECES;
-    const int st_row = tid / PPR, st_col = (tid % PPR) * 16;
-    const int st_off_k = DQ ? swz_store_off<D>(st_row, st_col) : st_row * PITCH + st_col;
-    const int st_off_v = DQ ? C::OFF_V + st_row * PITCH + st_col : C::OFF_TR + st_row * C::TPITCH + st_col;
-    u32x4 st_k = {0u, 0u, 0u, 0u}, st_v = {0u, 0u, 0u, 0u};
+    // ---- ring staging: direct-to-LDS loads, wave w moves chunk w of the K1 tile and of the V1 tile (D = 64: four
+    // chunks per tile, waves 0-3 stage)
+    using RT = typename C::RT;
+    const bool stager = wave < RT::NCH;
+    const int st_row = RT::st_row(wave % RT::NCH, lane), st_col = RT::st_col(lane);
     int n_load = 0, u_load = 0;
-    // address = tile base (uniform) + this thread's row and column (32 bits); only the diagonal tile can
+    // address = tile base (uniform) + this lane's row and column (32 bits); only the diagonal tile can
     // reach past the last row, so only it needs a clamped row
     const int st_row_diag = i0 + st_row < N ? st_row : N - 1 - i0;
     const uint32_t so_k = (uint32_t)(st_row * (int)p.k1.sn + st_col), so_v = (uint32_t)(st_row * (int)p.v1.sn + st_col);
     const uint32_t so_k_diag = (uint32_t)(st_row_diag * (int)p.k1.sn + st_col), so_v_diag = (uint32_t)(st_row_diag * (int)p.v1.sn + st_col);
+    const uint32_t lds_chunk = (uint32_t)(uintptr_t)lds + (wave % RT::NCH) * RT::CP;
     auto issue_loads = [&]() {
         const int t = t_lo + n_load;
         const char *kb = k1g + (int64_t)(32 * t) * p.k1.sn;
         const char *vb = v1g + (int64_t)(32 * t) * p.v1.sn;
         if (stager) {
-            st_k = ld_global16(kb + (t == t_hi ? so_k_diag : so_k));
-            st_v = ld_global16(vb + (t == t_hi ? so_v_diag : so_v));
+            const uint32_t dst = lds_chunk + (u_load & 1) * C::BUF;
+            load_to_lds16(kb, t == t_hi ? so_k_diag : so_k, dst);
+            load_to_lds16(vb, t == t_hi ? so_v_diag : so_v, dst + C::OFF_V);
         }
         ++u_load;
         n_load = (n_load == NT - 1) ? 0 : n_load + 1;
     };
-    auto write_stage = [&](int buf_off) {
-        if (stager) {
-            *reinterpret_cast<u32x4 *>(lds + buf_off + st_off_k) = st_k;
-            *reinterpret_cast<u32x4 *>(lds + buf_off + st_off_v) = st_v;
-        }
-    };
-    const int r_lane = c * PITCH + 16 * hf;                              // row-major fragment: row c, pieces 2*kk + hf
-    const int t_lane = C::OFF_TR + tr_lane_off<D, C::TPITCH>(lane);      // transposed fragment, per-lane part
-    const SwzLane<D> swz_lane(lane);                                      // DQ: fragments of the swizzled K1 tile
+    const int r_lane = RT::row_lane(lane);            // row fragment: row c, pieces 2*kk + hf
+    const int t_lane = RT::tr_lane(lane);             // transposed fragment, per-lane part
 
     // ---- fp32 rows shared by the workgroup, zeroed; q/do rows and the k2/v2 rows of the first round staged
     float *dqs = reinterpret_cast<float *>(lds + C::DQS);
@@ -231,24 +223,17 @@ __global__ __launch_bounds__(512) void bwd_q_kernel(KParams p, float *ws, int ha
         }
     };
 
-    // ring protocol: step u lives in buffer u & 1; it is written at the end of step u - 1 (every wave
-    // has passed the barrier of step u - 1, so none still reads that buffer) from registers loaded
-    // one step earlier, and published by the barrier of step u
+    // ring protocol: step u lives in buffer u & 1.  Its transfer starts behind the barrier of step u - 1 (every
+    // wave has then finished step u - 2, the last reader of that buffer) and is awaited before the barrier of step u.
     issue_loads();
-    write_stage(0);
-    if (U > 1) issue_loads();
     int u = 0;
-    auto stage_ahead = [&]() {
-        if (u + 1 < U) {
-            write_stage(((u + 1) & 1) * C::BUF);
-            if (u_load < U) issue_loads();
-        }
-        ++u;
+    auto open_step = [&]() {
+        if (stager) wait_loads<0>();
+        __syncthreads();
+        if (u + 1 < U) issue_loads();
     };
 
-    f32x16 neg_delta;          // DQ: -delta_i in every element (one query row per lane column)
-#pragma unroll
-    for (int rr = 0; rr < 16; ++rr) neg_delta[rr] = -dl;
+    const f32x16 neg_delta = splat16(-dl);      // DQ: -delta_i in every element (one query row per lane column)
     f32x16 acc[DT];            // G^T (DQ) or T^T (DV) of the running offset
     u32x4 A[KS];
     u32x4 Bv[DQ ? KS : 1];
@@ -283,61 +268,75 @@ __global__ __launch_bounds__(512) void bwd_q_kernel(KParams p, float *ws, int ha
         const float nl = col_ok ? -lse2 : -INFINITY;  // where the logit chains start
 
         for (int n = 0; n < NT; ++n) {
-            __syncthreads();
+            open_step();
             if (wave_on) {
                 const char *sub = lds + (u & 1) * C::BUF;
                 const int t = t_lo + n;
-                f32x16 X;
+                f32x16 X = splat16(nl);
                 if (t == t_hi || n < n_head) {
                     const char *mk = lds + C::MASKS + (t == t_hi ? 0 : 1 + n) * C::MASK + lane * 16;
 #pragma unroll
                     for (int qq = 0; qq < 4; ++qq) {
                         const float4 m4 = *reinterpret_cast<const float4 *>(mk + qq * 1024);
-                        X[4 * qq] = m4.x + nl;
-                        X[4 * qq + 1] = m4.y + nl;
-                        X[4 * qq + 2] = m4.z + nl;
-                        X[4 * qq + 3] = m4.w + nl;
+                        X[4 * qq] += m4.x;
+                        X[4 * qq + 1] += m4.y;
+                        X[4 * qq + 2] += m4.z;
+                        X[4 * qq + 3] += m4.w;
                     }
-                } else {
-#pragma unroll
-                    for (int rr = 0; rr < 16; ++rr) X[rr] = nl;
                 }
-#pragma unroll
-                for (int kk = 0; kk < KS; ++kk) X = mfma32(DQ ? swz_lane.row_frag(sub, kk) : ld_lds16(sub + r_lane + 32 * kk), A[kk], X);
-                f32x16 dP;
-                if constexpr (DQ) {
-                    // the chain starts from a register set that holds -delta_i: dP - delta costs no VALU work
-                    dP = mfma32(ld_lds16(sub + C::OFF_V + r_lane), Bv[0], neg_delta);
-#pragma unroll
-                    for (int kk = 1; kk < KS; ++kk) dP = mfma32(ld_lds16(sub + C::OFF_V + r_lane + 32 * kk), Bv[kk], dP);
-                }
+                // The operand fragments of the step form one stream: the K1 row fragments of the logit chain, (DQ) the
+                // V1 row fragments of the dP chain, then the transposed fragments of the accumulating products.  A
+                // window of W fragments is kept in flight: behind every MFMA the fragment W places further down the
+                // stream is requested (a scheduling fence keeps it there), so a read has W MFMAs of time to
+                // arrive and no chain waits for LDS.
+                constexpr int W = 3;
+                constexpr int NROW = DQ ? 2 * KS : KS;          // row fragments
+                constexpr int NFR = NROW + 2 * DT;              // ... and transposed ones
+                const char *kb = sub + r_lane, *vb = sub + C::OFF_V + r_lane;
+                const char *tb = sub + (DQ ? 0 : C::OFF_V) + t_lane;      // DQ: G^T += K1^T dS^T;  DV: T^T += V1^T P^T
+                auto fragment = [&](auto idx) {
+                    constexpr int s = decltype(idx)::value;
+                    if constexpr (s < KS) return RT::row_frag(kb, s);
+                    else if constexpr (s < NROW) return RT::row_frag(vb, s - KS);
+                    else return RT::tr_frag(tb, (s - NROW) / DT, (s - NROW) % DT);
+                };
+                u32x4 f[W];
+                static_for<0, W>([&](auto s) { f[s] = fragment(s); });
+                f32x16 dP = neg_delta;      // DQ: the chain starts from -delta_i, so dP - delta costs no VALU work
+                __builtin_amdgcn_sched_barrier(0);
+                static_for<0, NROW>([&](auto sc_) {
+                    constexpr int s = decltype(sc_)::value;
+                    if constexpr (s < KS) X = mfma32(f[s % W], A[s], X);
+                    else dP = mfma32(f[s % W], Bv[DQ ? s - KS : 0], dP);
+                    f[s % W] = fragment(std::integral_constant<int, s + W>{});
+                    __builtin_amdgcn_sched_barrier(0);
+                });
+                // weights of the first 16 tile rows, their products, the weights of the other 16 rows between them
                 u32x4 pb[2];
-#pragma unroll
-                for (int rr = 0; rr < 16; rr += 2) {
-                    float p0 = fast_exp2(X[rr]);
-                    float p1 = fast_exp2(X[rr + 1]);
+                auto weights = [&](int rr) {
+                    float p0 = fast_exp2(X[rr]), p1 = fast_exp2(X[rr + 1]);
                     if constexpr (DQ) {
                         p0 *= dP[rr];
                         p1 *= dP[rr + 1];
                     }
                     pb[rr >> 3][(rr & 7) >> 1] = pack_bf16(p0, p1);
-                }
+                };
 #pragma unroll
-                for (int k2s = 0; k2s < 2; ++k2s)
+                for (int rr = 0; rr < 8; rr += 2) weights(rr);
+                __builtin_amdgcn_sched_barrier(0);
+                static_for<0, 2 * DT>([&](auto sc_) {
+                    constexpr int s = decltype(sc_)::value;     // k2s = s / DT, dt = s % DT
+                    acc[s % DT] = mfma32(f[(NROW + s) % W], pb[s / DT], acc[s % DT]);
+                    if constexpr (NROW + s + W < NFR) f[(NROW + s) % W] = fragment(std::integral_constant<int, NROW + s + W>{});
+                    if constexpr (s < DT) {
+                        // (DT = 4: one pair of weights per MFMA; DT = 2: two pairs)
 #pragma unroll
-                    for (int dt = 0; dt < DT; ++dt) {
-                        u32x4 fr;
-                        if constexpr (DQ) {
-                            fr = swz_lane.tr_frag(sub, k2s, dt);
-                        } else {
-                            const u32x2 lo = lds_read_tr<D, C::TPITCH>(sub + t_lane, 16 * k2s, 32 * dt);
-                            const u32x2 hi = lds_read_tr<D, C::TPITCH>(sub + t_lane, 16 * k2s + 8, 32 * dt);
-                            fr = (u32x4){lo[0], lo[1], hi[0], hi[1]};
-                        }
-                        acc[dt] = mfma32(fr, pb[k2s], acc[dt]);
+                        for (int x = 0; x < 4 / DT; ++x) weights(8 + 2 * ((4 / DT) * s + x));
                     }
+                    __builtin_amdgcn_sched_barrier(0);
+                });
             }
-            stage_ahead();
+            ++u;
         }
 
         // ---- round end: add into the shared fp32 rows, one d-slice per wave and phase

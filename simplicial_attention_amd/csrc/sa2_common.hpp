@@ -12,6 +12,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 namespace sa2 {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
@@ -43,6 +45,15 @@ struct KParams {
     float scale;          // softmax scale
     float scale_log2e;    // scale * log2(e)
 };
+
+// compile-time loop: f(integral_constant<int, B>) ... f(integral_constant<int, E - 1>)
+template <int B, int E, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+    if constexpr (B < E) {
+        f(std::integral_constant<int, B>{});
+        static_for<B + 1, E>(f);
+    }
+}
 
 __device__ __forceinline__ float as_f32(uint32_t u) { return __builtin_bit_cast(float, u); }
 __device__ __forceinline__ uint32_t as_u32(float f) { return __builtin_bit_cast(uint32_t, f); }

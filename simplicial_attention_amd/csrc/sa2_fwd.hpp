@@ -42,15 +42,10 @@ struct FwdCfg {
     static constexpr int DT = D / 32;
     static constexpr int PITCH = tile_pitch<D>();     // staged q / k2 / v2 rows
     static constexpr int TILE = 32 * PITCH;
-    // K1 / V1 ring tiles are written by direct-to-LDS loads: one wave instruction moves 64 pieces of 16 bytes to
-    // 1 KiB of consecutive LDS, a "chunk" of RPC rows.  Inside a chunk the 64-byte segments of the rows are
-    // interleaved, [segment][row][64 bytes], and chunks start 1040 bytes apart: the 16 rows that a quarter of a
-    // row-fragment read touches, and the 4 rows x 64 bytes of a transposed read, then cover all 64 banks.
-    static constexpr int NSEG = D * 2 / 64;           // 64-byte segments per row
-    static constexpr int RPC = 16 / NSEG;             // rows per chunk
-    static constexpr int NCH = 32 / RPC;              // chunks per tile
-    static constexpr int CP = 1040;                   // chunk pitch
-    static constexpr int DTILE = NCH * CP;
+    // K1 / V1 ring tiles are written by direct-to-LDS loads (layout: DmaTile)
+    using RT = DmaTile<D>;
+    static constexpr int RPC = RT::RPC, NCH = RT::NCH, CP = RT::CP;
+    static constexpr int DTILE = RT::BYTES;
     static constexpr int BUF = 2 * DTILE;             // one ring buffer: a K1 tile and a V1 tile
     static constexpr int NBUF = 4;
     static constexpr int RING = NBUF * BUF;
@@ -64,38 +59,10 @@ struct FwdCfg {
     static constexpr int MASKS = V2S + KSLOTS * PITCH; // additive masks (0 / -inf) of the diagonal tile and of up to two lower-edge tiles
     static constexpr int MASK = 16 * 64 * 4;          // one table: [4 quarters][64 lanes][4 floats]
     static constexpr int LDS = MASKS + 3 * MASK;
-    // byte offset of element (row, d) inside a ring tile
-    static constexpr int ring_off(int row, int d) {
-        return (row / RPC) * CP + (d / 32) * (RPC * 64) + (row % RPC) * 64 + (d % 32) * 2;
-    }
     static_assert(RING - CP < 65536, "the LDS address of a direct load travels in 16 bits of M0");
     static constexpr int PPR = D / 8;                 // 16-byte pieces per row
     static constexpr int PIECES = 32 * PPR;           // ... per tile
 };
-
-// One direct-to-LDS load: lane l of the wave fetches the 16 bytes at base + offset_l and they land at LDS address
-// lds_addr + 16 l (both base and lds_addr are wave-uniform).  Counted by vmcnt like any global load; written as
-// assembly so that the compiler does not order the kernel's ordinary LDS reads behind it - the kernel waits for
-// the transfer itself (wait_loads) before the barrier that publishes the tile.
-__device__ __forceinline__ void load_to_lds16(const char *base, uint32_t lane_offset, uint32_t lds_addr) {
-    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_offset), "s"(base), "s"(lds_addr) : "memory");   // (m0 is reserved: the compiler keeps nothing in it across statements)
-}
-// sixteen registers holding x (each element is pinned to a register of its own: left to itself the compiler
-// copies a whole undefined tuple first and then overwrites fifteen of its registers)
-__device__ __forceinline__ f32x16 splat16(float x) {
-    f32x16 r;
-#pragma unroll
-    for (int e = 0; e < 16; ++e) {
-        float t = x;
-        asm("" : "+v"(t));
-        r[e] = t;
-    }
-    return r;
-}
-template <int N_LEFT>
-__device__ __forceinline__ void wait_loads() {
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N_LEFT) : "memory");
-}
 
 template <int D>
 __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
@@ -139,8 +106,7 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
     // ---- ring staging: direct-to-LDS loads, wave w moves chunk(s) w of the K1 tile and of the V1 tile.  Lane p of a
     // chunk load fetches row (p / 4) % RPC, segment p / (4 RPC), piece p % 4 of the segment
     const bool stager = wave < C::NCH;                           // D = 64: four chunks per tile, waves 0-3 stage
-    const int st_row = (wave % C::NCH) * C::RPC + (lane >> 2) % C::RPC;
-    const int st_col = (lane / (4 * C::RPC)) * 64 + (lane & 3) * 16;
+    const int st_row = C::RT::st_row(wave % C::NCH, lane), st_col = C::RT::st_col(lane);
     int n_load = 0;                                   // sequence index (within the round) of the next load
     int b_load = 0;                                   // ring buffer of the next load
     // address = tile base (uniform, on the scalar unit) + this lane's row and column (32 bits); only
@@ -161,9 +127,9 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
         b_load = (b_load == (C::NBUF - 1) * C::BUF) ? 0 : b_load + C::BUF;
     };
     // K1 fragment kk of row c: segment kk / 2, pieces 2 (kk % 2) + hf
-    const int k_lane = (c / C::RPC) * C::CP + (c % C::RPC) * 64 + 16 * hf;
+    const int k_lane = C::RT::row_lane(lane);
     // V1 transposed read: the lane's 8 bytes of row 4 hf + (lane % 16) / 4, d = 16 (lane & 1) + 8 (lane / 16 % 2) + 4 (lane % 4 / 2)
-    const int v_lane = C::DTILE + C::ring_off(4 * hf + ((lane & 15) >> 2), 16 * (lane & 1) + 8 * ((lane >> 4) & 1) + 4 * ((lane & 3) >> 1));
+    const int v_lane = C::DTILE + C::RT::tr_lane(lane);
 
     // ---- shared output accumulator and exchange areas
     float *acc_sh = reinterpret_cast<float *>(lds + C::RING);              // [32][APITCH]
@@ -291,20 +257,10 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
         };
         // fragment reads of a step: the V1 fragments of the tile behind its logit chain, the K1 fragments of
         // the next tile in front of the value chain (they arrive behind it and the barrier)
-        auto load_vf = [&]() {
-            const char *vbase = lds + b_cur + v_lane;
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                for (int k2s = 0; k2s < 2; ++k2s) {
-                    vf[dt][k2s][0] = lds_read_tr<D, 0>(vbase + C::ring_off(16 * k2s, 32 * dt), 0, 0);
-                    vf[dt][k2s][1] = lds_read_tr<D, 0>(vbase + C::ring_off(16 * k2s + 8, 32 * dt), 0, 0);
-                }
-        };
         auto load_kf = [&](int buf_off) {
             const char *kbase = lds + buf_off + k_lane;
 #pragma unroll
-            for (int kk = 0; kk < KS; ++kk) kf[kk] = ld_lds16(kbase + (kk >> 1) * (C::RPC * 64) + (kk & 1) * 32);
+            for (int kk = 0; kk < KS; ++kk) kf[kk] = ld_lds16(kbase + C::RT::row_imm(kk));
         };
         // The fragment reads of a step sit between its MFMAs, a scheduling fence behind every MFMA and its reads
         // keeps them there: the V1 fragments of the tile along its logit chain, the K1 fragments of the next tile
@@ -316,7 +272,7 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
                 const int k2s = m / DT, dt = m % DT;
                 u32x4 v = {vf[dt][k2s][0][0], vf[dt][k2s][0][1], vf[dt][k2s][1][0], vf[dt][k2s][1][1]};
                 T[dt] = mfma32(v, pb[k2s], T[dt]);
-                if (next_kf) kf[m] = ld_lds16(kbase + (m >> 1) * (C::RPC * 64) + (m & 1) * 32);
+                if (next_kf) kf[m] = ld_lds16(kbase + C::RT::row_imm(m));
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
@@ -327,8 +283,8 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
             for (int kk = 0; kk < KS; ++kk) {
                 X = mfma32(kf[kk], A[kk], X);
                 const int k2s = kk / DT, dt = kk % DT;
-                vf[dt][k2s][0] = lds_read_tr<D, 0>(vbase + C::ring_off(16 * k2s, 32 * dt), 0, 0);
-                vf[dt][k2s][1] = lds_read_tr<D, 0>(vbase + C::ring_off(16 * k2s + 8, 32 * dt), 0, 0);
+                vf[dt][k2s][0] = lds_read_tr<D, 0>(vbase + C::RT::tr_imm(16 * k2s, 32 * dt), 0, 0);
+                vf[dt][k2s][1] = lds_read_tr<D, 0>(vbase + C::RT::tr_imm(16 * k2s + 8, 32 * dt), 0, 0);
                 __builtin_amdgcn_sched_barrier(0);
             }
         };

@@ -84,4 +84,68 @@ struct SwzLane {
     }
 };
 
+// ---- tiles written by direct-to-LDS loads (global_load_lds_dwordx4)
+//
+// One wave instruction moves 64 pieces of 16 bytes to 1 KiB of consecutive LDS, a "chunk" of RPC rows of a
+// [32 rows][D] bf16 tile.  Which piece of global memory a lane fetches is free, so inside a chunk the 64-byte
+// segments of the rows are interleaved, [segment][row][64 bytes], and chunks start 1040 bytes apart: the 16 rows
+// that a quarter of a row-fragment read (ds_read_b128) touches, and the 4 rows x 64 bytes of a transposed read
+// (ds_read_b64_tr_b16), then cover all 64 banks.  The same tile serves both kinds of reads.
+template <int D>
+struct DmaTile {
+    static constexpr int NSEG = D * 2 / 64;           // 64-byte segments per row
+    static constexpr int RPC = 16 / NSEG;             // rows per chunk
+    static constexpr int NCH = 32 / RPC;              // chunks per tile
+    static constexpr int CP = 1040;                   // chunk pitch
+    static constexpr int BYTES = NCH * CP;
+    // byte offset of element (row, d)
+    __host__ __device__ static constexpr int off(int row, int d) {
+        return (row / RPC) * CP + (d / 32) * (RPC * 64) + (row % RPC) * 64 + (d % 32) * 2;
+    }
+    // staging: row and byte column that lane `lane` fetches for chunk `ch`
+    __device__ static int st_row(int ch, int lane) { return ch * RPC + (lane >> 2) % RPC; }
+    __device__ static int st_col(int lane) { return (lane / (4 * RPC)) * 64 + (lane & 3) * 16; }
+    // row fragment kk of row c (k-slots d = 16 kk + 8 hf .. + 7): per-lane part + immediate
+    __device__ static int row_lane(int lane) { return off(lane & 31, 0) + 16 * (lane >> 5); }
+    __host__ __device__ static constexpr int row_imm(int kk) { return (kk >> 1) * (RPC * 64) + (kk & 1) * 32; }
+    // transposed fragment (see lds_read_tr): per-lane part + immediate for (row_base multiple of 8, d_base multiple of 32)
+    __device__ static int tr_lane(int lane) {
+        return off(4 * (lane >> 5) + ((lane & 15) >> 2), 16 * (lane & 1) + 8 * ((lane >> 4) & 1) + 4 * ((lane & 3) >> 1));
+    }
+    __host__ __device__ static constexpr int tr_imm(int row_base, int d_base) { return off(row_base, d_base); }
+    __device__ static u32x4 row_frag(const char *tile_lane, int kk) { return ld_lds16(tile_lane + row_imm(kk)); }
+    __device__ static u32x4 tr_frag(const char *tile_lane, int k2s, int dt) {
+        const u32x2 lo = lds_read_tr<D, 0>(tile_lane + tr_imm(16 * k2s, 32 * dt), 0, 0);
+        const u32x2 hi = lds_read_tr<D, 0>(tile_lane + tr_imm(16 * k2s + 8, 32 * dt), 0, 0);
+        return (u32x4){lo[0], lo[1], hi[0], hi[1]};
+    }
+};
+
+// One direct-to-LDS load: lane l of the wave fetches the 16 bytes at base + offset_l and they land at LDS address
+// lds_addr + 16 l (base and lds_addr are wave-uniform; the LDS address travels in 16 bits of M0).  Counted by
+// vmcnt like any global load; written as assembly so that the compiler does not order the kernel's ordinary LDS
+// reads behind it - a kernel waits for the transfer itself (wait_loads) before the barrier that publishes the tile.
+__device__ __forceinline__ void load_to_lds16(const char *base, uint32_t lane_offset, uint32_t lds_addr) {
+    // (m0 is reserved: the compiler keeps nothing in it across statements)
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(lane_offset), "s"(base), "s"(lds_addr) : "memory");
+}
+// waits until at most N_LEFT of this wave's vector-memory operations are in flight
+template <int N_LEFT>
+__device__ __forceinline__ void wait_loads() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N_LEFT) : "memory");
+}
+
+// sixteen registers holding x (each element is pinned to a register of its own: left to itself the compiler
+// copies a whole undefined tuple first and then overwrites fifteen of its registers)
+__device__ __forceinline__ f32x16 splat16(float x) {
+    f32x16 r;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) {
+        float t = x;
+        asm("" : "+v"(t));
+        r[e] = t;
+    }
+    return r;
+}
+
 }  // namespace sa2
