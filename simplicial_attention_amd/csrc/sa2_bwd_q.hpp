@@ -289,7 +289,7 @@ __global__ __launch_bounds__(512) void bwd_q_kernel(KParams p, float *ws, int ha
                 // window of W fragments is kept in flight: behind every MFMA the fragment W places further down the
                 // stream is requested (a scheduling fence keeps it there), so a read has W MFMAs of time to
                 // arrive and no chain waits for LDS.
-                constexpr int W = 3;
+                constexpr int W = 4;
                 constexpr int NROW = DQ ? 2 * KS : KS;          // row fragments
                 constexpr int NFR = NROW + 2 * DT;              // ... and transposed ones
                 const char *kb = sub + r_lane, *vb = sub + C::OFF_V + r_lane;
