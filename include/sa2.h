@@ -58,7 +58,7 @@ typedef struct sa2_problem {
     int32_t kv_heads;   /* key/value heads, divides heads */
     int32_t dim_head;   /* 64 or 128 */
     int32_t w1;         /* window of the first key/value set  (reference default 512) */
-    int32_t w2;         /* window of the second key/value set (reference default 32), <= 64 */
+    int32_t w2;         /* window of the second key/value set (reference default 32), any value >= 1 */
     int32_t causal;     /* must be 1 */
     float   scale;      /* softmax scale, dim_head^-0.5 in the reference (:735) */
     int32_t dtype;      /* sa2_dtype of the activations */
@@ -94,8 +94,8 @@ int sa2_version(void);
 /* Message of the last failing call on this thread ("" if none). */
 const char *sa2_last_error(void);
 
-/* 1 if the kernels cover this configuration (dim_head 64 or 128, w2 <= 64, bf16), else 0.
- * Replaces the silent limits of the reference (HEAD_DIM fixed to 64, w2 <= 32:
+/* 1 if the kernels cover this configuration (dim_head 64 or 128, any w1 >= 1 and w2 >= 1, bf16),
+ * else 0.  Replaces the silent limits of the reference (HEAD_DIM fixed to 64, w2 <= 32:
  * triton_two_simplicial_attention.py:51,291,508,586). */
 int sa2_supported(int32_t dim_head, int32_t w1, int32_t w2, int32_t dtype);
 
@@ -122,7 +122,9 @@ int sa2_bwd_delta(const sa2_problem *prob, const sa2_tensor *out, const sa2_tens
 /* Bytes of device workspace the backward needs for this problem (fp32 partial rows of
  * dK2/dV2, one block per 32-row query tile); -1 if the problem is invalid.  The
  * reference has no counterpart: its five fp32 gradient buffers of
- * triton_two_simplicial_attention.py:853-857 play the same role. */
+ * triton_two_simplicial_attention.py:853-857 play the same role.  The first half holds the
+ * dK2 rows, the second half the dV2 rows: a backward call that is given the forward's saved
+ * partials (sa2_saved) touches only the first half and accepts half this size. */
 int64_t sa2_bwd_workspace_bytes(const sa2_problem *prob);
 
 /* dQ, dK2, dV2.  Replaces both passes of two_simplicial_attn_bwd_kv2q_kernel
@@ -130,8 +132,8 @@ int64_t sa2_bwd_workspace_bytes(const sa2_problem *prob);
  * dk2/dv2 :680-683, :695, :702-707).  One kernel owns the query rows (dQ complete,
  * dK2/dV2 as partial rows in the workspace), a second one sums the partial rows and
  * the query heads of a group.  No atomics; results are bitwise reproducible.
- * saved may be NULL; if it holds what sa2_fwd wrote for these inputs (and w2 <= 32),
- * dV2 is formed from it instead of from a recomputation of the attention weights. */
+ * saved may be NULL; if it holds what sa2_fwd wrote for these inputs, dV2 is formed from it
+ * instead of from a recomputation of the attention weights. */
 int sa2_bwd_dq_dkv2(const sa2_problem *prob,
                     const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
                     const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *dout,

@@ -263,10 +263,13 @@ int sa2_bwd_dq_dkv2(const sa2_problem *prob, const sa2_tensor *q, const sa2_tens
     SA2_TRY(check_tensor(dv2, "dv2"));
     if (!workspace) return fail(SA2_ERR_NULL_POINTER, "workspace is NULL");
     if ((reinterpret_cast<uintptr_t>(workspace) & 15) != 0) return fail(SA2_ERR_ALIGNMENT, "workspace must be 16-byte aligned");
-    const int64_t need = sa2_bwd_workspace_bytes(prob);
+    // the dK2 partial rows are the first half of the workspace, the dV2 partial rows the second: with saved
+    // forward partials dV2 needs none
+    const bool saved_given = saved != nullptr;
+    const int64_t need = sa2_bwd_workspace_bytes(prob) / (saved_given ? 2 : 1);
     if (workspace_bytes < need)
-        return fail(SA2_ERR_BAD_SHAPE, "workspace of %lld bytes is smaller than the %lld bytes sa2_bwd_workspace_bytes() asks for",
-                    (long long)workspace_bytes, (long long)need);
+        return fail(SA2_ERR_BAD_SHAPE, "workspace of %lld bytes is smaller than the %lld bytes this call needs (sa2_bwd_workspace_bytes()%s)",
+                    (long long)workspace_bytes, (long long)need, saved_given ? " / 2 with saved partials" : "");
     k.dq = dev(dq);
     k.dk2 = dev(dk2);
     k.dv2 = dev(dv2);
