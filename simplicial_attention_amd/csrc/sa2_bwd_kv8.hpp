@@ -320,6 +320,26 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     build(nb, 0);
     next_pair(nb);
 
+    // A chain of N MFMAs whose LDS operand fragments are requested W places ahead: behind every MFMA the
+    // fragment W places further down is read (a scheduling fence keeps it there), so the chain waits for
+    // LDS once, at its start, instead of before every MFMA.  frag(integral_constant<s>) reads fragment s,
+    // step(integral_constant<s>, fragment) issues MFMA s.
+    auto mfma_stream = [&](auto n_tag, auto frag, auto step) {
+        constexpr int NF = decltype(n_tag)::value;
+        constexpr int W = 3;
+        u32x4 f[W];
+        static_for<0, W>([&](auto s_) { f[s_] = frag(s_); });
+        __builtin_amdgcn_sched_barrier(0);
+        static_for<0, NF>([&](auto s_) {
+            constexpr int x = decltype(s_)::value;
+            step(s_, f[x % W]);
+            if constexpr (x + W < NF) f[x % W] = frag(std::integral_constant<int, x + W>{});
+            __builtin_amdgcn_sched_barrier(0);
+        });
+    };
+    using NChain = std::integral_constant<int, KS>;
+    using NProd = std::integral_constant<int, 2 * DT>;
+
     if constexpr (SPLIT) {
         // The two roles run separate loops with the same barrier sequence (per pair: tiles
         // complete; [new query tile: rows replaced]; P in LDS), so that neither loop carries
@@ -360,10 +380,13 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                             X[4 * a4 + 2] = l4.z;
                             X[4 * a4 + 3] = l4.w;
                         }
-#pragma unroll
-                        for (int kk = 0; kk < KS; ++kk) X = mfma32(swz_lane.row_frag(buf + L::AS, kk), k1f[kk], X);
-                        if (!full) {
-                            const int base = 32 * it + 4 * hf - j;   // i - j for register 0
+                        mfma_stream(NChain{}, [&](auto kk) { return swz_lane.row_frag(buf + L::AS, kk); },
+                                    [&](auto kk, const u32x4 &fr) { X = mfma32(fr, k1f[kk], X); });
+                        if (__builtin_expect(!full, 0)) {
+                            // (the tile reaches over an edge of the first window; the distance is made opaque so that
+                            // none of this is computed ahead of the branch)
+                            int base = 32 * it + 4 * hf - j;         // i - j for register 0
+                            asm volatile("" : "+v"(base));
 #pragma unroll
                             for (int rr = 0; rr < 16; ++rr) {
                                 const bool ok = (unsigned)(base + 8 * (rr >> 2) + (rr & 3)) < (unsigned)p.w1;
@@ -377,10 +400,8 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                         *reinterpret_cast<u32x4 *>(px + e * 2048) = pb[0];
                         *reinterpret_cast<u32x4 *>(px + e * 2048 + 1024) = pb[1];
                         if (e == 0) {
-#pragma unroll
-                            for (int k2s = 0; k2s < 2; ++k2s)
-#pragma unroll
-                                for (int dt = 0; dt < DT; ++dt) acc[dt] = mfma32(swz_lane.tr_frag(buf + L::BS, k2s, dt), pb[k2s], acc[dt]);
+                            mfma_stream(NProd{}, [&](auto x) { return swz_lane.tr_frag(buf + L::BS, x / DT, x % DT); },
+                                        [&](auto x, const u32x4 &fr) { acc[x % DT] = mfma32(fr, pb[x / DT], acc[x % DT]); });
                         } else {
                             pb_late[0] = pb[0];
                             pb_late[1] = pb[1];
@@ -392,10 +413,8 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                 if (on) {
                     // the S waves now have MFMA and VALU work of their own; this evens out the two halves
                     const char *buf = pair + L::STEP;
-#pragma unroll
-                    for (int k2s = 0; k2s < 2; ++k2s)
-#pragma unroll
-                        for (int dt = 0; dt < DT; ++dt) acc[dt] = mfma32(swz_lane.tr_frag(buf + L::BS, k2s, dt), pb_late[k2s], acc[dt]);
+                    mfma_stream(NProd{}, [&](auto x) { return swz_lane.tr_frag(buf + L::BS, x / DT, x % DT); },
+                                [&](auto x, const u32x4 &fr) { acc[x % DT] = mfma32(fr, pb_late[x / DT], acc[x % DT]); });
                 }
                 if (more) {
                     build(nb, (s + 1) & 1);                     // the P waves' share of the next pair's tiles
@@ -426,9 +445,8 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                             dPe[e][4 * a4 + 2] = d4.z;
                             dPe[e][4 * a4 + 3] = d4.w;
                         }
-#pragma unroll
-                        for (int kk = 0; kk < KS; ++kk) dPe[e] = mfma32(swz_lane.row_frag(buf + L::BS, kk), k1f[kk], dPe[e]);
-                        __builtin_amdgcn_sched_barrier(0);
+                        mfma_stream(NChain{}, [&](auto kk) { return swz_lane.row_frag(buf + L::BS, kk); },
+                                    [&](auto kk, const u32x4 &fr) { dPe[e] = mfma32(fr, k1f[kk], dPe[e]); });
                     }
                 }
                 // the MFMA chains first, the build after them: measured faster than the other order
@@ -450,11 +468,8 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                             for (int w = 0; w < 4; ++w)
                                 pb[hh][w] = pack_bf16(bf16_lo(pq[w]) * dPe[e][8 * hh + 2 * w], bf16_hi(pq[w]) * dPe[e][8 * hh + 2 * w + 1]);
                         }
-#pragma unroll
-                        for (int k2s = 0; k2s < 2; ++k2s)
-#pragma unroll
-                            for (int dt = 0; dt < DT; ++dt) acc[dt] = mfma32(swz_lane.tr_frag(buf + L::AS, k2s, dt), pb[k2s], acc[dt]);
-                        __builtin_amdgcn_sched_barrier(0);
+                        mfma_stream(NProd{}, [&](auto x) { return swz_lane.tr_frag(buf + L::AS, x / DT, x % DT); },
+                                    [&](auto x, const u32x4 &fr) { acc[x % DT] = mfma32(fr, pb[x / DT], acc[x % DT]); });
                     }
                 }
             }
