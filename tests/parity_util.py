@@ -9,11 +9,13 @@ Two input distributions are used, each with the tolerance that was stated for it
   small, so the absolute part is loose; the relative Frobenius error (<= 1e-2) is
   the binding check.
 * ``std = 1`` (unit-variance logits, the inputs of the reference's own
-  tests/test_triton.py): the reference's tolerances, atol 3e-2 on the output
-  (tests/test_triton.py:104) and atol 5e-2 on the gradients (:111-115), plus the same
-  relative Frobenius bound; additionally at most 1e-4 of the elements may fall
-  outside the build-target formula (bf16 rounding of the MFMA operands q*k2 and
-  do*v2 gives individual gradient elements an error of about 2.5e-2 at this scale).
+  tests/test_triton.py): the same criterion (every element, no allowance), the same
+  relative Frobenius bound, and the reference's own tolerances on top, atol 3e-2 on the
+  output (tests/test_triton.py:104) and atol 5e-2 on the gradients (:111-115).
+  One case is judged by the reference's absolute tolerances alone
+  (``reference_atol_only``): windows of one entry with unit-variance inputs, where the
+  exact dq, dk1, dk2 are zero and what the kernels return is the bf16 rounding of the
+  operand do*v2 in dS = P (dP - delta), about 3e-2.
 """
 import torch
 
@@ -66,7 +68,8 @@ def compare(name, got, ref):
     return dict(name=name, max_abs=float(err.max()), ref_max=float(ref.abs().max()), rel_fro=rel_f, bad=bad)
 
 
-def check_all(got_out, got_grads, ref_out, ref_grads, rel_fro_limit=1e-2, unit_variance=False, verbose=True):
+def check_all(got_out, got_grads, ref_out, ref_grads, rel_fro_limit=1e-2, unit_variance=False, verbose=True,
+              reference_atol_only=False):
     rows = [compare(n, g, r) for n, g, r in zip(NAMES, (got_out, *got_grads), (ref_out, *ref_grads))]
     if verbose:
         for r in rows:
@@ -76,8 +79,7 @@ def check_all(got_out, got_grads, ref_out, ref_grads, rel_fro_limit=1e-2, unit_v
         if unit_variance:
             atol = 3e-2 if r['name'] == 'out' else 5e-2
             assert r['max_abs'] <= atol, f"{r['name']}: max abs error {r['max_abs']:.3e} > {atol}"
-            assert r['bad'] <= 1e-4 * ref.numel(), f"{r['name']}: {r['bad']} elements outside {ATOL} + {RTOL}|ref|"
-        else:
+        if not reference_atol_only:
             assert r['bad'] == 0, f"{r['name']}: {r['bad']} elements outside |x-ref| <= {ATOL} + {RTOL}|ref| (max abs {r['max_abs']:.3e})"
         assert r['rel_fro'] <= rel_fro_limit, f"{r['name']}: relative Frobenius error {r['rel_fro']:.3e} > {rel_fro_limit}"
     return rows
