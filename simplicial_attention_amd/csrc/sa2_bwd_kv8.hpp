@@ -466,11 +466,10 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
             X[4 * a4 + 2] = l4.z;
             X[4 * a4 + 3] = l4.w;
         }
-#pragma unroll
-        for (int kk = 0; kk < KS; ++kk) X = mfma32(row_frag(buf + L::AS, kk), k1f[kk], X);
+        mfma_stream(NChain{}, [&](auto kk) { return row_frag(buf + L::AS, kk); },
+                    [&](auto kk, const u32x4 &fr) { X = mfma32(fr, k1f[kk], X); });
         f32x16 dP;
         if constexpr (DK) {
-            __builtin_amdgcn_sched_barrier(0);        // keeps the two sets of fragments from being live together
             // the accumulator starts at -delta_i (stored negated by the build): dP - delta costs no VALU work
 #pragma unroll
             for (int a4 = 0; a4 < 4; ++a4) {
@@ -480,12 +479,13 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                 dP[4 * a4 + 2] = d4.z;
                 dP[4 * a4 + 3] = d4.w;
             }
-#pragma unroll
-            for (int kk = 0; kk < KS; ++kk) dP = mfma32(row_frag(buf + L::BS, kk), v1f[kk], dP);
+            mfma_stream(NChain{}, [&](auto kk) { return row_frag(buf + L::BS, kk); },
+                        [&](auto kk, const u32x4 &fr) { dP = mfma32(fr, v1f[kk], dP); });
         }
         const bool full = (jw + 31 <= 32 * it) && (jw + p.w1 > 32 * it + 31);
-        if (!full) {
-            const int base = 32 * it + 4 * hf - j;   // i - j for register 0
+        if (__builtin_expect(!full, 0)) {
+            int base = 32 * it + 4 * hf - j;         // i - j for register 0
+            asm volatile("" : "+v"(base));           // (keeps the edge-tile code behind the branch)
 #pragma unroll
             for (int rr = 0; rr < 16; ++rr) {
                 const bool ok = (unsigned)(base + 8 * (rr >> 2) + (rr & 3)) < (unsigned)p.w1;
@@ -505,14 +505,11 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
             }
             pb[rr >> 3][(rr & 7) >> 1] = pack_bf16(p0, p1);
         }
-#pragma unroll
-        for (int k2s = 0; k2s < 2; ++k2s)
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt) {
-                if constexpr (DK) acc[dt] = mfma32(tr_frag(buf + L::AS, k2s, dt), pb[k2s], acc[dt]);
-                else acc[dt] = mfma32(tr_frag(buf + L::BS, k2s, dt), pb[k2s], acc[dt]);
-                if constexpr (TWO) acc2[dt] = mfma32(tr_frag(buf + L::BS, k2s, dt), pv[k2s], acc2[dt]);
-            }
+        mfma_stream(NProd{}, [&](auto x) { return tr_frag(buf + (DK ? L::AS : L::BS), x / DT, x % DT); },
+                    [&](auto x, const u32x4 &fr) { acc[x % DT] = mfma32(fr, pb[x / DT], acc[x % DT]); });
+        if constexpr (TWO)
+            mfma_stream(NProd{}, [&](auto x) { return tr_frag(buf + L::BS, x / DT, x % DT); },
+                        [&](auto x, const u32x4 &fr) { acc2[x % DT] = mfma32(fr, pv[x / DT], acc2[x % DT]); });
     }
 
     // ---- add the two groups of every slab and store
