@@ -4,8 +4,7 @@
 // slab.  The workgroup walks pairs of "steps" (query head of the group, 32-row query tile,
 // offset dlt); a pair holds the offsets 2m and 2m+1 of one query tile.  The q/do rows of a
 // query tile and the 63 k2/v2 rows its offsets (at most 32) can reach are staged in LDS
-// once per staging unit (query tile, block of 32 offsets), the q/do rows as fp32 (unpacked once,
-// q times scale log2 e); from them the 512 threads build A = q*k2 and B = do*v2 of both steps
+// once per tile; from them the 512 threads build A = q*k2 and B = do*v2 of both steps
 // once per pair (A carries scale log2(e), so S is the exponent's variable part and dK1 comes out
 // times scale log2(e): it is stored times ln 2).  With P = exp2(S - lse log2(e)):
 //   S = A K1^T,  dP = B V1^T,  dS = P (dP - delta),  dK1^T += A^T dS,  dV1^T += B^T P.
@@ -23,10 +22,10 @@
 //                  dS = P dP and dK1^T += A^T dS.  Two contractions per wave and offset,
 //                  one operand build per pair, no final reduction.
 // (MODEs kKvDk / kKvDv, the two-pass forms that each recompute S, are not instantiated.)
+// Every MFMA chain requests its LDS fragments three places ahead (mfma_stream).
 // S and dP read row fragments of the A and B tiles (ds_read_b128), the accumulating
-// products read transposed fragments (ds_read_b64_tr_b16); the tiles are stored once, in the
-// chunked layout of DmaTile (sa2_lds.hpp), which serves both kinds of reads without bank
-// conflicts.  Every MFMA chain requests its fragments three places ahead (mfma_stream).
+// products read transposed fragments (ds_read_b64_tr_b16).  A tile that is read both ways
+// is stored once, in the swizzled layout of sa2_lds.hpp.
 #pragma once
 
 #include <type_traits>
@@ -43,12 +42,20 @@ struct Kv8Cfg {
     static_assert(MODE == kKvBoth || MODE == kKvSplit, "only the single-kernel forms are built");
     static constexpr bool DK = MODE != kKvDv;         // dK1 is produced (needs dP, delta, V1)
     static constexpr bool DV = MODE != kKvDk;         // dV1 is produced
-    // step buffer: [A][B][lse][delta]; the operand tiles use the chunked, segment-interleaved layout of DmaTile, which
-    // serves row fragments and transposed fragments alike (a thread's 16-byte piece goes to DmaTile::off(row, d))
-    using OT = DmaTile<D>;
+    static constexpr int PITCH = tile_pitch<D>();
+    static constexpr int TILE = 32 * PITCH;
+    static constexpr int TPITCH = tr_pitch<D>();
+    static constexpr int TRT = 32 * TPITCH;
+    // step buffer: dk1:  [A swizzled][B row-major][lse][delta]
+    //              dv1:  [A row-major][B transposed-read][lse]
+    //              both: [A swizzled][B swizzled][lse][delta]
+    static constexpr bool A_SWZ = DK;                 // A is read both ways
+    static constexpr bool B_SWZ = DK && DV;           // B is read both ways
+    static constexpr int A_PITCH = A_SWZ ? TPITCH : PITCH;
+    static constexpr int B_PITCH = DV ? TPITCH : PITCH;
     static constexpr int AS = 0;
-    static constexpr int BS = OT::BYTES;
-    static constexpr int LSE = BS + OT::BYTES;
+    static constexpr int BS = 32 * A_PITCH;
+    static constexpr int LSE = BS + 32 * B_PITCH;
     static constexpr int DEL = LSE + 32 * 4;
     static constexpr int STEP = DEL + 32 * 4;
     static constexpr int PAIR = 2 * STEP;
@@ -56,22 +63,20 @@ struct Kv8Cfg {
     // staged rows of the current query tile (unpadded, read lane-linear by the builders)
     static constexpr int HALO = 31;
     static constexpr int KROWS = 32 + HALO;           // k in [32 it - 31, 32 it + 31]
-    static constexpr int RP = 2 * D;                  // bytes per staged k2/v2 row (bf16)
-    static constexpr int RPF = 4 * D;                 // bytes per staged q/do row: fp32, unpacked once per query tile (q times scale log2 e)
+    static constexpr int RP = 2 * D;                  // bytes per staged row
     static constexpr int QS = TILES;
-    static constexpr int DOS = QS + 32 * RPF;
-    static constexpr int K2S = DOS + 32 * RPF;
+    static constexpr int DOS = QS + 32 * RP;
+    static constexpr int K2S = DOS + 32 * RP;
     static constexpr int V2S = K2S + KROWS * RP;
     static constexpr int LSES = V2S + KROWS * RP;     // 32 floats lse * log2e, 32 floats delta
     static constexpr int PX = LSES + 64 * 4;          // kKvSplit: packed P of [slab][offset of the pair], 2 KiB each
-    static constexpr int LDS_LOOP = PX + (MODE == kKvSplit ? 4 * 2 * 2048 : 0);
+    static constexpr int LDS = PX + (MODE == kKvSplit ? 4 * 2 * 2048 : 0);
     static constexpr int NROWP = (64 + 2 * KROWS) * (D / 8);        // 16-byte pieces of the staged rows
     static constexpr int RPT = (NROWP + 511) / 512;                 // ... per thread
     static constexpr int RPITCH = D + 4;              // floats per row of the final reduction
     static constexpr int LPT = 32 * D / 8 / 256;      // 16-byte pieces per thread and tensor
     static constexpr int RED = 128 * RPITCH * 4;      // bytes of one output's final reduction
-    static constexpr int LDS_RED = (MODE == kKvBoth ? 2 : 1) * RED;     // the final reduction reuses the loop's LDS (everything else is dead by then)
-    static constexpr int LDS = LDS_LOOP > LDS_RED ? LDS_LOOP : LDS_RED;
+    static_assert((MODE == kKvBoth ? 2 : 1) * RED <= LDS, "final reduction must fit (everything else is dead by then)");
 };
 
 template <int D, int MODE>
@@ -80,6 +85,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     using L = Kv8Cfg<D, MODE>;
     constexpr bool DK = L::DK, TWO = MODE == kKvBoth, SPLIT = MODE == kKvSplit;
     static_assert(!TWO || D == 64, "both accumulators fit two waves per SIMD at D = 64 only");
+    constexpr int PITCH = L::PITCH;
     __shared__ __attribute__((aligned(16))) char lds[L::LDS];
 
     const int N = p.N;
@@ -129,11 +135,24 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     const int wit_hi = ((jw + 31 + p.w1 - 1 < N - 1) ? jw + 31 + p.w1 - 1 : N - 1) / 32;
     const float c2 = p.scale_log2e;
     // per-lane parts of the fragment addresses: plain row-major / transposed-read tiles, swizzled tiles
-    using OT = typename L::OT;
-    const int r_lane = OT::row_lane(lane);
-    const int t_lane = OT::tr_lane(lane);
-    auto row_frag = [&](const char *image, int kk) { return OT::row_frag(image + r_lane, kk); };
-    auto tr_frag = [&](const char *image, int k2s, int dt) { return OT::tr_frag(image + t_lane, k2s, dt); };
+    const int r_lane = c * PITCH + 16 * hf;
+    const int t_lane = tr_lane_off<D, L::TPITCH>(lane);
+    const SwzLane<D> swz_lane(lane);
+    auto row_frag = [&](const char *image, auto swz, int kk) {
+        if constexpr (decltype(swz)::value) return swz_lane.row_frag(image, kk);
+        else return ld_lds16(image + r_lane + 32 * kk);
+    };
+    auto tr_frag = [&](const char *image, auto swz, int k2s, int dt) {
+        if constexpr (decltype(swz)::value) {
+            return swz_lane.tr_frag(image, k2s, dt);
+        } else {
+            const u32x2 lo2 = lds_read_tr<D, L::TPITCH>(image + t_lane, 16 * k2s, 32 * dt);
+            const u32x2 hi2 = lds_read_tr<D, L::TPITCH>(image + t_lane, 16 * k2s + 8, 32 * dt);
+            return (u32x4){lo2[0], lo2[1], hi2[0], hi2[1]};
+        }
+    };
+    using ASwz = std::integral_constant<bool, L::A_SWZ>;
+    using BSwz = std::integral_constant<bool, L::B_SWZ>;
 
     // ---- pair iterator (g, it, blk, m): offsets 32 blk + 2m and 32 blk + 2m + 1 of query tile `it`, query head g
     // of the group.  (it, blk) is the staging unit: the q/do rows of the tile and the 63 k2/v2 rows that the 32
@@ -202,19 +221,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
         for (int x = 0; x < L::RPT; ++x) {
             const int pc = x * 512 + tid;
             if (pc >= L::NROWP) break;
-            if (pc < 64 * PPR) {
-                // a q or dO piece: eight fp32 values (q carries scale log2 e from here on)
-                const int row = pc / PPR, col = (pc % PPR) * 16;
-                const float f = row < 32 ? c2 : 1.f;
-                float4 lo, hi;
-                lo.x = bf16_lo(rows[x][0]) * f; lo.y = bf16_hi(rows[x][0]) * f; lo.z = bf16_lo(rows[x][1]) * f; lo.w = bf16_hi(rows[x][1]) * f;
-                hi.x = bf16_lo(rows[x][2]) * f; hi.y = bf16_hi(rows[x][2]) * f; hi.z = bf16_lo(rows[x][3]) * f; hi.w = bf16_hi(rows[x][3]) * f;
-                float4 *dst = reinterpret_cast<float4 *>(lds + L::QS + row * L::RPF + col * 2);     // (the dO rows follow the q rows)
-                dst[0] = lo;
-                dst[1] = hi;
-            } else {
-                *reinterpret_cast<u32x4 *>(lds + L::K2S + (pc - 64 * PPR) * 16) = rows[x];         // k2, v2 rows are contiguous
-            }
+            *reinterpret_cast<u32x4 *>(lds + L::QS + pc * 16) = rows[x];     // q, do, k2, v2 rows are contiguous
         }
         if (tid < 32) {
             reinterpret_cast<float *>(lds + L::LSES)[tid] = r_lse;
@@ -225,10 +232,26 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     // ---- operand build.  A tile has 32 * D/8 pieces of 16 bytes: 512 at D = 128, one per
     // thread, and a thread builds its piece of A and of B; 256 at D = 64, where threads 0-255
     // build A and threads 256-511 build B.  Either way a thread builds ITS piece for both steps
-    // of the pair from one read of its (already unpacked) q or dO piece.
+    // of the pair, so the q (dO) piece is read and unpacked once for two products.
+    // dv1 pass: the thread's q and dO pieces stay unpacked in registers for the whole query
+    // tile (the dk1 pass has no registers to spare and unpacks them once per pair)
     constexpr int PIECES = 32 * PPR;
     constexpr bool BOTH = PIECES == 512;
+    constexpr bool KEEP = MODE == kKvDv && BOTH;
     const int b_row = (tid % PIECES) / PPR, b_col = (tid % PPR) * 16;
+    float qx[8], ox[8];
+    auto unpack_own = [&]() {
+        const int row = b_row, col = b_col;
+        const u32x4 fq = ld_lds16(lds + L::QS + row * L::RP + col);
+        const u32x4 fo = ld_lds16(lds + L::DOS + row * L::RP + col);
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            qx[2 * w] = bf16_lo(fq[w]) * c2;
+            qx[2 * w + 1] = bf16_hi(fq[w]) * c2;
+            ox[2 * w] = bf16_lo(fo[w]);
+            ox[2 * w + 1] = bf16_hi(fo[w]);
+        }
+    };
     auto build = [&](const Pair &s, int buf) {
         const int row = b_row, col = b_col;
         const int dmax = dmax_of(s.it, s.blk);
@@ -236,11 +259,8 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
         const int dl0 = 2 * s.m;                                   // never dead
         const bool dead1 = dl0 + 1 > dmax;
         const int dl1 = dead1 ? dl0 : dl0 + 1;
-        const int o_tile = OT::off(row, col / 2);
-        auto product = [&](int xs, int bs, int tile_off) {        // xs: q or dO rows (fp32), bs: k2 or v2 rows (bf16)
-            const float4 x0 = *reinterpret_cast<const float4 *>(lds + xs + row * L::RPF + col * 2);
-            const float4 x1 = *reinterpret_cast<const float4 *>(lds + xs + row * L::RPF + col * 2 + 16);
-            const float xv[8] = {x0.x, x0.y, x0.z, x0.w, x1.x, x1.y, x1.z, x1.w};
+        auto product = [&](const float (&xv)[8], int bs, auto is_a) {   // xv: q (times scale log2 e) or dO piece, bs: k2 or v2 rows
+            constexpr bool IS_A = decltype(is_a)::value;
             u32x4 r0, r1;
             const u32x4 f0 = ld_lds16(lds + bs + (row - dl0 + L::HALO) * L::RP + col);
             const u32x4 f1 = ld_lds16(lds + bs + (row - dl1 + L::HALO) * L::RP + col);
@@ -249,12 +269,34 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                 r0[w] = pack_bf16(xv[2 * w] * bf16_lo(f0[w]), xv[2 * w + 1] * bf16_hi(f0[w]));
                 r1[w] = pack_bf16(xv[2 * w] * bf16_lo(f1[w]), xv[2 * w + 1] * bf16_hi(f1[w]));
             }
-            *reinterpret_cast<u32x4 *>(stage + tile_off + o_tile) = r0;
-            *reinterpret_cast<u32x4 *>(stage + L::STEP + tile_off + o_tile) = r1;
+            constexpr bool SWZ = IS_A ? L::A_SWZ : L::B_SWZ;
+            const int o = (IS_A ? L::AS : L::BS) + (SWZ ? swz_store_off<D>(row, col) : row * (IS_A ? L::A_PITCH : L::B_PITCH) + col);
+            *reinterpret_cast<u32x4 *>(stage + o) = r0;
+            *reinterpret_cast<u32x4 *>(stage + L::STEP + o) = r1;
         };
-        if (BOTH || tid < PIECES) product(L::QS, L::K2S, L::AS);
-        if constexpr (BOTH) __builtin_amdgcn_sched_barrier(0);   // one product at a time: there are no registers for both
-        if (BOTH || tid >= PIECES) product(L::DOS, L::V2S, L::BS);
+        if constexpr (KEEP) {
+            product(qx, L::K2S, std::true_type{});
+            product(ox, L::V2S, std::false_type{});
+        } else {
+            float xv[8];
+            auto unpack = [&](int xs, float f) {
+                const u32x4 fx = ld_lds16(lds + xs + row * L::RP + col);
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    xv[2 * w] = bf16_lo(fx[w]) * f;
+                    xv[2 * w + 1] = bf16_hi(fx[w]) * f;
+                }
+            };
+            if (BOTH || tid < PIECES) {
+                unpack(L::QS, c2);
+                product(xv, L::K2S, std::true_type{});
+            }
+            if constexpr (BOTH) __builtin_amdgcn_sched_barrier(0);   // one product at a time: the dk1 pass has no registers for both
+            if (BOTH || tid >= PIECES) {
+                unpack(L::DOS, 1.f);
+                product(xv, L::V2S, std::false_type{});
+            }
+        }
         if (tid < 64) {
             const int e = tid >> 5, r = tid & 31;
             const int i = 32 * s.it + r;
@@ -274,6 +316,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     write_rows();
     if (rw.g < p.G) issue_rows(rw);
     __syncthreads();
+    if constexpr (KEEP) unpack_own();
     build(nb, 0);
     next_pair(nb);
 
@@ -337,7 +380,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                             X[4 * a4 + 2] = l4.z;
                             X[4 * a4 + 3] = l4.w;
                         }
-                        mfma_stream(NChain{}, [&](auto kk) { return row_frag(buf + L::AS, kk); },
+                        mfma_stream(NChain{}, [&](auto kk) { return swz_lane.row_frag(buf + L::AS, kk); },
                                     [&](auto kk, const u32x4 &fr) { X = mfma32(fr, k1f[kk], X); });
                         if (__builtin_expect(!full, 0)) {
                             // (the tile reaches over an edge of the first window; the distance is made opaque so that
@@ -357,7 +400,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                         *reinterpret_cast<u32x4 *>(px + e * 2048) = pb[0];
                         *reinterpret_cast<u32x4 *>(px + e * 2048 + 1024) = pb[1];
                         if (e == 0) {
-                            mfma_stream(NProd{}, [&](auto x) { return tr_frag(buf + L::BS, x / DT, x % DT); },
+                            mfma_stream(NProd{}, [&](auto x) { return swz_lane.tr_frag(buf + L::BS, x / DT, x % DT); },
                                         [&](auto x, const u32x4 &fr) { acc[x % DT] = mfma32(fr, pb[x / DT], acc[x % DT]); });
                         } else {
                             pb_late[0] = pb[0];
@@ -370,7 +413,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                 if (on) {
                     // the S waves now have MFMA and VALU work of their own; this evens out the two halves
                     const char *buf = pair + L::STEP;
-                    mfma_stream(NProd{}, [&](auto x) { return tr_frag(buf + L::BS, x / DT, x % DT); },
+                    mfma_stream(NProd{}, [&](auto x) { return swz_lane.tr_frag(buf + L::BS, x / DT, x % DT); },
                                 [&](auto x, const u32x4 &fr) { acc[x % DT] = mfma32(fr, pb_late[x / DT], acc[x % DT]); });
                 }
                 if (more) {
@@ -402,7 +445,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                             dPe[e][4 * a4 + 2] = d4.z;
                             dPe[e][4 * a4 + 3] = d4.w;
                         }
-                        mfma_stream(NChain{}, [&](auto kk) { return row_frag(buf + L::BS, kk); },
+                        mfma_stream(NChain{}, [&](auto kk) { return swz_lane.row_frag(buf + L::BS, kk); },
                                     [&](auto kk, const u32x4 &fr) { dPe[e] = mfma32(fr, k1f[kk], dPe[e]); });
                     }
                 }
@@ -425,7 +468,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                             for (int w = 0; w < 4; ++w)
                                 pb[hh][w] = pack_bf16(bf16_lo(pq[w]) * dPe[e][8 * hh + 2 * w], bf16_hi(pq[w]) * dPe[e][8 * hh + 2 * w + 1]);
                         }
-                        mfma_stream(NProd{}, [&](auto x) { return tr_frag(buf + L::AS, x / DT, x % DT); },
+                        mfma_stream(NProd{}, [&](auto x) { return swz_lane.tr_frag(buf + L::AS, x / DT, x % DT); },
                                     [&](auto x, const u32x4 &fr) { acc[x % DT] = mfma32(fr, pb[x / DT], acc[x % DT]); });
                     }
                 }
@@ -445,7 +488,8 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                 next_unit(rw);
                 if (rw.g < p.G) issue_rows(rw);
                 __syncthreads();
-                        }
+                if constexpr (KEEP) unpack_own();
+            }
             build(nb, (s + 1) & 1);
             next_pair(nb);
         }
@@ -466,7 +510,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
             X[4 * a4 + 2] = l4.z;
             X[4 * a4 + 3] = l4.w;
         }
-        mfma_stream(NChain{}, [&](auto kk) { return row_frag(buf + L::AS, kk); },
+        mfma_stream(NChain{}, [&](auto kk) { return row_frag(buf + L::AS, ASwz{}, kk); },
                     [&](auto kk, const u32x4 &fr) { X = mfma32(fr, k1f[kk], X); });
         f32x16 dP;
         if constexpr (DK) {
@@ -479,7 +523,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                 dP[4 * a4 + 2] = d4.z;
                 dP[4 * a4 + 3] = d4.w;
             }
-            mfma_stream(NChain{}, [&](auto kk) { return row_frag(buf + L::BS, kk); },
+            mfma_stream(NChain{}, [&](auto kk) { return row_frag(buf + L::BS, BSwz{}, kk); },
                         [&](auto kk, const u32x4 &fr) { dP = mfma32(fr, v1f[kk], dP); });
         }
         const bool full = (jw + 31 <= 32 * it) && (jw + p.w1 > 32 * it + 31);
@@ -505,10 +549,14 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
             }
             pb[rr >> 3][(rr & 7) >> 1] = pack_bf16(p0, p1);
         }
-        mfma_stream(NProd{}, [&](auto x) { return tr_frag(buf + (DK ? L::AS : L::BS), x / DT, x % DT); },
-                    [&](auto x, const u32x4 &fr) { acc[x % DT] = mfma32(fr, pb[x / DT], acc[x % DT]); });
+        if constexpr (DK)
+            mfma_stream(NProd{}, [&](auto x) { return tr_frag(buf + L::AS, ASwz{}, x / DT, x % DT); },
+                        [&](auto x, const u32x4 &fr) { acc[x % DT] = mfma32(fr, pb[x / DT], acc[x % DT]); });
+        else
+            mfma_stream(NProd{}, [&](auto x) { return tr_frag(buf + L::BS, BSwz{}, x / DT, x % DT); },
+                        [&](auto x, const u32x4 &fr) { acc[x % DT] = mfma32(fr, pb[x / DT], acc[x % DT]); });
         if constexpr (TWO)
-            mfma_stream(NProd{}, [&](auto x) { return tr_frag(buf + L::BS, x / DT, x % DT); },
+            mfma_stream(NProd{}, [&](auto x) { return tr_frag(buf + L::BS, BSwz{}, x / DT, x % DT); },
                         [&](auto x, const u32x4 &fr) { acc2[x % DT] = mfma32(fr, pv[x / DT], acc2[x % DT]); });
     }
 
