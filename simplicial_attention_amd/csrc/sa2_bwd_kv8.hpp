@@ -308,6 +308,47 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
             if constexpr (DK) reinterpret_cast<float *>(st + L::DEL)[r] = valid ? -reinterpret_cast<const float *>(lds + L::LSES)[32 + r] : 0.f;
         }
     };
+    // kKvSplit: a quarter of the pair's operand tiles - 256 pieces (16 rows) of A or of B for both offsets - built
+    // by the 256 threads of one wave group.  The two groups do not take equal shares of a pair's build: measured
+    // per pair, the S waves are busy longer than the P waves in both halves of a pair (1428 + 1500 against 1700 + 330
+    // cycles of chain and softmax work), so the P waves build three quarters and the S waves one.
+    auto build_quarter = [&](const Pair &s, int buf, auto is_a, int half) {
+        constexpr bool IS_A = decltype(is_a)::value;
+        const int pc = half * 256 + (tid & 255);
+        const int row = pc / PPR, col = (pc % PPR) * 16;
+        const int dmax = dmax_of(s.it, s.blk);
+        char *stage = lds + buf * L::PAIR;
+        const int dl0 = 2 * s.m;                                   // never dead
+        const int dl1 = dl0 + 1 > dmax ? dl0 : dl0 + 1;
+        const int bs = IS_A ? L::K2S : L::V2S;
+        const u32x4 fx = ld_lds16(lds + (IS_A ? L::QS : L::DOS) + row * L::RP + col);
+        const u32x4 f0 = ld_lds16(lds + bs + (row - dl0 + L::HALO) * L::RP + col);
+        const u32x4 f1 = ld_lds16(lds + bs + (row - dl1 + L::HALO) * L::RP + col);
+        const float f = IS_A ? c2 : 1.f;
+        u32x4 r0, r1;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) {
+            const float xl = bf16_lo(fx[w]) * f, xh = bf16_hi(fx[w]) * f;
+            r0[w] = pack_bf16(xl * bf16_lo(f0[w]), xh * bf16_hi(f0[w]));
+            r1[w] = pack_bf16(xl * bf16_lo(f1[w]), xh * bf16_hi(f1[w]));
+        }
+        const int o = (IS_A ? L::AS : L::BS) + swz_store_off<D>(row, col);
+        *reinterpret_cast<u32x4 *>(stage + o) = r0;
+        *reinterpret_cast<u32x4 *>(stage + L::STEP + o) = r1;
+    };
+    // the -lse / -delta start values of the pair's chains (64 threads of the P group)
+    auto build_tables = [&](const Pair &s, int buf) {
+        if (tid < 64) {
+            const int dmax = dmax_of(s.it, s.blk);
+            const int e = tid >> 5, r = tid & 31;
+            const int i = 32 * s.it + r;
+            const int dlt = 2 * s.m + e;
+            const bool valid = dlt <= dmax && i < N && i - 32 * s.blk - dlt >= 0;
+            char *st = lds + buf * L::PAIR + e * L::STEP;
+            reinterpret_cast<float *>(st + L::LSE)[r] = valid ? -reinterpret_cast<const float *>(lds + L::LSES)[r] : -INFINITY;
+            reinterpret_cast<float *>(st + L::DEL)[r] = valid ? -reinterpret_cast<const float *>(lds + L::LSES)[32 + r] : 0.f;
+        }
+    };
     Pair nb = {0, it_begin, 0, 0};   // next pair to build
     Pair cur = {0, it_begin, 0, 0};  // pair being computed
     Pair rw = {0, it_begin, 0, 0};   // staging unit whose rows are loaded next
@@ -409,6 +450,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                         __builtin_amdgcn_sched_barrier(0);      // one offset at a time: its fragments are dead before the next one's are loaded
                     }
                 }
+                if (more) build_quarter(nb, (s + 1) & 1, std::true_type{}, 0);
                 __syncthreads();                                // P of the pair is in LDS
                 if (on) {
                     // the S waves now have MFMA and VALU work of their own; this evens out the two halves
@@ -417,7 +459,10 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                                 [&](auto x, const u32x4 &fr) { acc[x % DT] = mfma32(fr, pb_late[x / DT], acc[x % DT]); });
                 }
                 if (more) {
-                    build(nb, (s + 1) & 1);                     // the P waves' share of the next pair's tiles
+                    build_quarter(nb, (s + 1) & 1, std::false_type{}, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                    build_quarter(nb, (s + 1) & 1, std::false_type{}, 1);
+                    build_tables(nb, (s + 1) & 1);
                     next_pair(nb);
                 }
             }
@@ -452,7 +497,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                 // the MFMA chains first, the build after them: measured faster than the other order
                 // (the P waves start the pair with MFMA work as well and then turn to their exponentials)
                 if (more) {
-                    build(nb, (s + 1) & 1);
+                    build_quarter(nb, (s + 1) & 1, std::true_type{}, 1);
                     next_pair(nb);
                 }
                 __syncthreads();                                // P of the pair is in LDS
