@@ -420,26 +420,40 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
                 if (hf == 0) p.m_save[srow_g] = fresh ? 0.f : M;
             }
             Mc = Mn;
-            const char *v2row = lds + C::V2S + slot * PITCH + 16 * hf * 2;
+            // the round's contribution of this wave, v2_{i-dlt} * T * g, is formed in place in T before the phases
+            // (nothing there depends on another wave), so that a phase is only: read the slice, add, write, barrier
+            {
+                const char *v2row = lds + C::V2S + slot * PITCH + 16 * hf * 2;
+#pragma unroll
+                for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+                    for (int half = 0; half < 2; ++half) {
+                        const u32x4 xv = ld_lds16(v2row + dt * 64 + half * 16);
+#pragma unroll
+                        for (int w = 0; w < 4; ++w) {
+                            T[dt][8 * half + 2 * w] *= bf16_lo(xv[w]) * g;
+                            T[dt][8 * half + 2 * w + 1] *= bf16_hi(xv[w]) * g;
+                        }
+                    }
+            }
             float *arow = acc_sh + c * C::APITCH + 16 * hf;
             auto add_slice = [&](auto slice_tag, bool first) {
                 constexpr int S = decltype(slice_tag)::value;     // slice: dt = S / 2, registers 8*(S%2) .. +7
                 constexpr int dt = S >> 1, r0 = 8 * (S & 1);
-                const u32x4 xv = ld_lds16(v2row + dt * 64 + r0 * 2);
                 float *dst = arow + 32 * dt + r0;
                 float4 a0 = *reinterpret_cast<float4 *>(dst), a1 = *reinterpret_cast<float4 *>(dst + 4);
                 if (first) {
                     a0.x *= fo; a0.y *= fo; a0.z *= fo; a0.w *= fo;
                     a1.x *= fo; a1.y *= fo; a1.z *= fo; a1.w *= fo;
                 }
-                a0.x += bf16_lo(xv[0]) * T[dt][r0] * g;
-                a0.y += bf16_hi(xv[0]) * T[dt][r0 + 1] * g;
-                a0.z += bf16_lo(xv[1]) * T[dt][r0 + 2] * g;
-                a0.w += bf16_hi(xv[1]) * T[dt][r0 + 3] * g;
-                a1.x += bf16_lo(xv[2]) * T[dt][r0 + 4] * g;
-                a1.y += bf16_hi(xv[2]) * T[dt][r0 + 5] * g;
-                a1.z += bf16_lo(xv[3]) * T[dt][r0 + 6] * g;
-                a1.w += bf16_hi(xv[3]) * T[dt][r0 + 7] * g;
+                a0.x += T[dt][r0];
+                a0.y += T[dt][r0 + 1];
+                a0.z += T[dt][r0 + 2];
+                a0.w += T[dt][r0 + 3];
+                a1.x += T[dt][r0 + 4];
+                a1.y += T[dt][r0 + 5];
+                a1.z += T[dt][r0 + 6];
+                a1.w += T[dt][r0 + 7];
                 *reinterpret_cast<float4 *>(dst) = a0;
                 *reinterpret_cast<float4 *>(dst + 4) = a1;
             };
