@@ -41,6 +41,32 @@ def test_fwd_bwd_matches_oracle(b, n, hq, hk, d, w1, w2, unit_variance):
     U.check_all(out, grads, ref_out, ref_grads, unit_variance=unit_variance)
 
 
+def _random_shapes(count, seed=1234):
+    import random
+    rng = random.Random(seed)
+    shapes = []
+    for _ in range(count):
+        d = rng.choice([64, 128])
+        hk = rng.choice([1, 2])
+        hq = hk * rng.choice([1, 2])
+        n = rng.choice([rng.randint(1, 40), rng.randint(33, 130), rng.randint(131, 420)])
+        w1 = rng.choice([rng.randint(1, 40), rng.randint(30, 140), rng.randint(100, 600)])
+        w2 = rng.choice([rng.randint(1, 9), rng.randint(8, 33), rng.randint(30, 80)])
+        shapes.append((rng.choice([1, 2]), n, hq, hk, d, w1, w2))
+    return shapes
+
+
+@pytest.mark.parametrize('b,n,hq,hk,d,w1,w2', _random_shapes(24))
+def test_seeded_random_shapes(b, n, hq, hk, d, w1, w2):
+    """A seeded draw of sequence lengths, windows, head counts and head dimensions (ragged tiles, windows
+    shorter and longer than the sequence, one to ten offset rounds, grouped heads)."""
+    print(f'\ncase b={b} n={n} hq={hq} hk={hk} d={d} w1={w1} w2={w2}', flush=True)
+    ins = U.make_inputs(b, n, hq, hk, d, seed=n * 7 + w1 * 3 + w2, std=d ** -0.5)
+    ref_out, _, ref_grads = U.oracle_fwd_bwd(*ins, w1, w2)
+    out, grads = U.hip_fwd_bwd(*ins, w1, w2)
+    U.check_all(out, grads, ref_out, ref_grads)
+
+
 def test_large_and_drifting_logits():
     """Logits that grow along the sequence by far more than 2^64 per window: exercises
     the paths of the forward that move the softmax reference point while accumulators
