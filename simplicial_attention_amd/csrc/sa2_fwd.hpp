@@ -2,26 +2,26 @@
 //
 // One workgroup owns 32 query rows of one (batch, head).  In round r wave w handles the
 // offset dlt = i - k = 8r + w (any second window: ceil(w2 / 8) rounds); all eight waves walk
-// the same 32-row K1/V1 tiles, which stream through a three-buffer LDS ring, one tile and
-// one barrier per step.  Per (offset, tile):
+// the same 32-row K1/V1 tiles, which stream through a four-buffer LDS ring (direct-to-LDS loads,
+// layout DmaTile of sa2_lds.hpp), one tile and one barrier per step.  Per (offset, tile):
 //     S^T = K1 A^T          A = q_i * k2_{i-dlt} * scale * log2(e)   (bf16, built once per offset)
 //     P^T = exp2(S^T - M_i)                 (the MFMA chain starts from -M_i: no VALU subtraction)
 //     T^T += V1^T P^T       (V1 fragments through ds_read_b64_tr_b16)
-// Measured on MI355X: a wave hides about four plain VALU instructions behind each of its own
-// 32x32x16 MFMAs and none beyond that, and a second wave on the SIMD fills the MFMA pipe while
-// the first one runs its exponentials - provided that phase is shorter than an MFMA phase.
+// Measured on MI355X: a 32x32x16 MFMA occupies the SIMD's issue port for about 15 of its 36-38
+// cycles and every other VALU instruction for about 4.9, from either wave of the SIMD: four to five
+// VALU instructions per MFMA hide behind it and none beyond that.
 // So the per-tile VALU work is kept to the exponentials, the bf16 packing and the row sums:
 //   - the softmax reference M of a row is fixed by the first tile of the wave's first offset
 //     (the diagonal tile, which every valid row attends) and moves only when a row sum says
 //     that weights grew beyond 2^90 (a branch that is almost never taken);
 //   - masks are applied on the diagonal tile and on the (at most two) tiles that the window's
 //     lower edge crosses; the tiles in between run without mask code;
-//   - the V1 fragments of a tile are requested when its logit chain has been issued and arrive
-//     behind the exponentials; the K1 fragments of the next tile are requested in front of the
-//     value chain and arrive behind it and the barrier.
+//   - fragment reads are spread between the MFMAs (a scheduling fence behind every MFMA and its reads):
+//     the V1 fragments of a tile along its logit chain, the K1 fragments of the next tile along the
+//     value chain.
 // The output accumulator is shared: an fp32 [32][D] LDS buffer relative to a common reference
 // Mc.  At the end of a round the waves publish their references, agree on Mc = max, and add
-// v2_{i-dlt} * T * 2^(M - Mc) in eight barrier-separated phases; in phase ph wave w owns the
+// v2_{i-dlt} * T * 2^(M - Mc) (formed in place in T first) in eight barrier-separated phases; in phase ph wave w owns the
 // d-slice (w + ph) mod 8, so concurrent waves never touch the same element and every element
 // sees its additions in a fixed order (bitwise reproducible, no atomics).
 // The k2/v2 rows live in a 64-row circular LDS buffer (row k in slot (k - i0) mod 64): a round
