@@ -461,7 +461,7 @@ int sa2_qkv_norm_bwd(const sa2_problem *prob, const void *qkv, int64_t row_strid
         hipLaunchKernelGGL(sa2::qkv_norm_bwd_kernel<64>, dim3(blocks), dim3(256), 0, s, np, groups);
     SA2_TRY(after_launch("qkv norm backward"));
     const int n = 5 * prob->dim_head;
-    hipLaunchKernelGGL(sa2::qkv_norm_dw_kernel, dim3((n + 255) / 256), dim3(256), 0, s, np.dw_part, dw, blocks, n);
+    hipLaunchKernelGGL(sa2::qkv_norm_dw_kernel, dim3((n + 15) / 16), dim3(256), 0, s, np.dw_part, dw, blocks, n);
     return after_launch("qkv norm weight gradients");
 }
 

@@ -84,7 +84,7 @@ __global__ __launch_bounds__(256) void qkv_norm_fwd_kernel(NormParams p) {
 // Weight gradients: a block walks groups of 256 / (D/8) head rows with a grid stride; every
 // (row slot, 8-element piece) thread keeps its own LDS accumulators per tensor, the block
 // adds the row slots in a fixed order and writes one partial [5][D]; qkv_norm_dw_kernel
-// adds the partials of the blocks in block order (bitwise reproducible, no atomics).
+// adds the partials of the blocks in a fixed order (bitwise reproducible, no atomics).
 template <int D>
 __global__ __launch_bounds__(256) void qkv_norm_bwd_kernel(NormParams p, int ngroups) {
     constexpr int LP = D / 8, RPB = 256 / LP;
@@ -142,13 +142,24 @@ __global__ __launch_bounds__(256) void qkv_norm_bwd_kernel(NormParams p, int ngr
     }
 }
 
-// dw[tensor][d] = sum over blocks of the partials, in block order; one thread per (tensor, d)
+// dw[tensor][d] = sum over blocks of the partials, in a fixed order.  A block of 256 threads owns 16 consecutive
+// outputs x = (tensor, d); thread (x, phase) adds the partials of the blocks phase, phase + 16, ... (the 16 threads of
+// a phase read 64 consecutive bytes of one partial), then the 16 phases of an output are added in phase order.
 __global__ __launch_bounds__(256) void qkv_norm_dw_kernel(const float *part, float *dw, int nblocks, int n /* 5 * D */) {
-    const int x = blockIdx.x * 256 + threadIdx.x;
-    if (x >= n) return;
+    __shared__ float red[16][17];
+    const int xl = threadIdx.x & 15, phase = threadIdx.x >> 4;
+    const int x = blockIdx.x * 16 + xl;
     float s = 0.f;
-    for (int b = 0; b < nblocks; ++b) s += part[(int64_t)b * n + x];
-    dw[x] = s;
+    if (x < n)
+        for (int b = phase; b < nblocks; b += 16) s += part[(int64_t)b * n + x];
+    red[phase][xl] = s;
+    __syncthreads();
+    if (phase == 0 && x < n) {
+        float t = 0.f;
+#pragma unroll
+        for (int q = 0; q < 16; ++q) t += red[q][xl];
+        dw[x] = t;
+    }
 }
 
 }  // namespace sa2
