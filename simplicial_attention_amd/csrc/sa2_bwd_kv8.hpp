@@ -20,7 +20,12 @@
 //                  pair, and it leaves the packed P in LDS.  Wave "S" holds the V1 rows and
 //                  the dK1 accumulator: dP - delta meanwhile, then (one barrier later)
 //                  dS = P dP and dK1^T += A^T dS.  Two contractions per wave and offset,
-//                  one operand build per pair, no final reduction.
+//                  one operand build per pair, no final reduction.  Both roles are software
+//                  pipelines: the VALU work (exponentials of one offset, dS of the next, the
+//                  quarters of the next pair's operand tiles) is cut into eight pieces that
+//                  are issued behind the eight MFMAs of a chain that does not depend on them.
+//                  The P waves build three quarters of the tiles, the S waves one (the S waves
+//                  are the busier ones behind the barrier).
 // (MODEs kKvDk / kKvDv, the two-pass forms that each recompute S, are not instantiated.)
 // Every MFMA chain requests its LDS fragments three places ahead (mfma_stream).
 // S and dP read row fragments of the A and B tiles (ds_read_b128), the accumulating
@@ -308,34 +313,6 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
             if constexpr (DK) reinterpret_cast<float *>(st + L::DEL)[r] = valid ? -reinterpret_cast<const float *>(lds + L::LSES)[32 + r] : 0.f;
         }
     };
-    // kKvSplit: a quarter of the pair's operand tiles - 256 pieces (16 rows) of A or of B for both offsets - built
-    // by the 256 threads of one wave group.  The two groups do not take equal shares of a pair's build: measured
-    // per pair, the S waves are busy longer than the P waves in both halves of a pair (1428 + 1500 against 1700 + 330
-    // cycles of chain and softmax work), so the P waves build three quarters and the S waves one.
-    auto build_quarter = [&](const Pair &s, int buf, auto is_a, int half) {
-        constexpr bool IS_A = decltype(is_a)::value;
-        const int pc = half * 256 + (tid & 255);
-        const int row = pc / PPR, col = (pc % PPR) * 16;
-        const int dmax = dmax_of(s.it, s.blk);
-        char *stage = lds + buf * L::PAIR;
-        const int dl0 = 2 * s.m;                                   // never dead
-        const int dl1 = dl0 + 1 > dmax ? dl0 : dl0 + 1;
-        const int bs = IS_A ? L::K2S : L::V2S;
-        const u32x4 fx = ld_lds16(lds + (IS_A ? L::QS : L::DOS) + row * L::RP + col);
-        const u32x4 f0 = ld_lds16(lds + bs + (row - dl0 + L::HALO) * L::RP + col);
-        const u32x4 f1 = ld_lds16(lds + bs + (row - dl1 + L::HALO) * L::RP + col);
-        const float f = IS_A ? c2 : 1.f;
-        u32x4 r0, r1;
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            const float xl = bf16_lo(fx[w]) * f, xh = bf16_hi(fx[w]) * f;
-            r0[w] = pack_bf16(xl * bf16_lo(f0[w]), xh * bf16_hi(f0[w]));
-            r1[w] = pack_bf16(xl * bf16_lo(f1[w]), xh * bf16_hi(f1[w]));
-        }
-        const int o = (IS_A ? L::AS : L::BS) + swz_store_off<D>(row, col);
-        *reinterpret_cast<u32x4 *>(stage + o) = r0;
-        *reinterpret_cast<u32x4 *>(stage + L::STEP + o) = r1;
-    };
     // the -lse / -delta start values of the pair's chains (64 threads of the P group)
     auto build_tables = [&](const Pair &s, int buf) {
         if (tid < 64) {
@@ -365,7 +342,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     // fragment W places further down is read (a scheduling fence keeps it there), so the chain waits for
     // LDS once, at its start, instead of before every MFMA.  frag(integral_constant<s>) reads fragment s,
     // step(integral_constant<s>, fragment) issues MFMA s.
-    auto mfma_stream = [&](auto n_tag, auto frag, auto step) {
+    auto mfma_stream2 = [&](auto n_tag, auto frag, auto step, auto side) {
         constexpr int NF = decltype(n_tag)::value;
         constexpr int W = 3;
         u32x4 f[W];
@@ -375,9 +352,11 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
             constexpr int x = decltype(s_)::value;
             step(s_, f[x % W]);
             if constexpr (x + W < NF) f[x % W] = frag(std::integral_constant<int, x + W>{});
+            side(s_);                    // independent VALU work issued behind MFMA s
             __builtin_amdgcn_sched_barrier(0);
         });
     };
+    auto mfma_stream = [&](auto n_tag, auto frag, auto step) { mfma_stream2(n_tag, frag, step, [](auto) {}); };
     using NChain = std::integral_constant<int, KS>;
     using NProd = std::integral_constant<int, 2 * DT>;
 
@@ -395,127 +374,184 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                 __syncthreads();
             }
         };
+        // A quarter of the next pair's operand tiles as eight pieces of VALU work that ride behind the MFMAs of a chain:
+        // load (three 16-byte LDS reads), piece 2w (q or dO pair w unpacked, product with the first offset's row),
+        // piece 2w + 1 (product with the second offset's row), store.
+        struct QB {
+            u32x4 fx, f0, f1, r0, r1;
+            float xl, xh;
+            char *dst;
+        };
+        auto qb_load = [&](QB &qb, const Pair &s, int buf, auto is_a, int half) {
+            constexpr bool IS_A = decltype(is_a)::value;
+            const int pc = half * 256 + (tid & 255);
+            const int row = pc / PPR, col = (pc % PPR) * 16;
+            const int dmax = dmax_of(s.it, s.blk);
+            const int dl0 = 2 * s.m;                                   // never dead
+            const int dl1 = dl0 + 1 > dmax ? dl0 : dl0 + 1;
+            const int bs = IS_A ? L::K2S : L::V2S;
+            qb.fx = ld_lds16(lds + (IS_A ? L::QS : L::DOS) + row * L::RP + col);
+            qb.f0 = ld_lds16(lds + bs + (row - dl0 + L::HALO) * L::RP + col);
+            qb.f1 = ld_lds16(lds + bs + (row - dl1 + L::HALO) * L::RP + col);
+            qb.dst = lds + buf * L::PAIR + (IS_A ? L::AS : L::BS) + swz_store_off<D>(row, col);
+        };
+        auto qb_piece = [&](QB &qb, auto k_, float f) {
+            constexpr int k = decltype(k_)::value, w = k >> 1;
+            if constexpr ((k & 1) == 0) {
+                qb.xl = bf16_lo(qb.fx[w]) * f;
+                qb.xh = bf16_hi(qb.fx[w]) * f;
+                qb.r0[w] = pack_bf16(qb.xl * bf16_lo(qb.f0[w]), qb.xh * bf16_hi(qb.f0[w]));
+            } else {
+                qb.r1[w] = pack_bf16(qb.xl * bf16_lo(qb.f1[w]), qb.xh * bf16_hi(qb.f1[w]));
+            }
+        };
+        auto qb_store = [&](QB &qb) {
+            *reinterpret_cast<u32x4 *>(qb.dst) = qb.r0;
+            *reinterpret_cast<u32x4 *>(qb.dst + L::STEP) = qb.r1;
+        };
+        static_assert(KS == 8 && 2 * DT == 8, "the pipelines pair eight pieces of VALU work with the eight MFMAs of a chain");
+        auto start_from = [&](f32x16 &X, const char *table) {
+#pragma unroll
+            for (int a4 = 0; a4 < 4; ++a4) {
+                const float4 l4 = *reinterpret_cast<const float4 *>(table + (8 * a4 + 4 * hf) * 4);
+                X[4 * a4] = l4.x;
+                X[4 * a4 + 1] = l4.y;
+                X[4 * a4 + 2] = l4.z;
+                X[4 * a4 + 3] = l4.w;
+            }
+        };
         if (pg == 0) {
-            // ---- P waves: S, P (left in LDS for the other wave of the slab), dV1^T += B^T P
+            // ---- P waves: S, P (left in LDS for the other wave of the slab), dV1^T += B^T P, three quarters of the build.
+            // Software pipeline: build quarter beside the first logit chain, the exponentials of the first offset beside the
+            // second logit chain, those of the second beside the first offset's dV1 products, two build quarters beside
+            // the second offset's dV1 products.
             for (int s = 0; s < npairs; ++s) {
                 const bool more = s + 1 < npairs;
                 open_pair(more);
-                const char *pair = lds + (s & 1) * L::PAIR;
+                const char *buf0 = lds + (s & 1) * L::PAIR, *buf1 = buf0 + L::STEP;
+                const int nbuf = (s + 1) & 1;
                 const int it = cur.it;
                 next_pair(cur);
                 const bool on = wave_active && it >= wit_lo && it <= wit_hi;
-                u32x4 pb_late[2];                               // P of the second offset: its dV1 products run after the barrier
-                if (on) {
-                    const bool full = (jw + 31 <= 32 * it) && (jw + p.w1 > 32 * it + 31);
+                const bool full = (jw + 31 <= 32 * it) && (jw + p.w1 > 32 * it + 31);
+                auto edge = [&](f32x16 &X) {
+                    if (__builtin_expect(!full, 0)) {
+                        // (the tile reaches over an edge of the first window; the distance is made opaque so that
+                        // none of this is computed ahead of the branch)
+                        int base = 32 * it + 4 * hf - j;         // i - j for register 0
+                        asm volatile("" : "+v"(base));
 #pragma unroll
-                    for (int e = 0; e < 2; ++e) {
-                        const char *buf = pair + e * L::STEP;
-                        // the chain starts from -lse_i log2(e) (stored negated by the build; -inf for dead rows), and A
-                        // carries scale * log2(e): the result is the exponent
-                        f32x16 X;
-#pragma unroll
-                        for (int a4 = 0; a4 < 4; ++a4) {
-                            const float4 l4 = *reinterpret_cast<const float4 *>(buf + L::LSE + (8 * a4 + 4 * hf) * 4);
-                            X[4 * a4] = l4.x;
-                            X[4 * a4 + 1] = l4.y;
-                            X[4 * a4 + 2] = l4.z;
-                            X[4 * a4 + 3] = l4.w;
+                        for (int rr = 0; rr < 16; ++rr) {
+                            const bool ok = (unsigned)(base + 8 * (rr >> 2) + (rr & 3)) < (unsigned)p.w1;
+                            X[rr] = ok ? X[rr] : -INFINITY;
                         }
-                        mfma_stream(NChain{}, [&](auto kk) { return swz_lane.row_frag(buf + L::AS, kk); },
-                                    [&](auto kk, const u32x4 &fr) { X = mfma32(fr, k1f[kk], X); });
-                        if (__builtin_expect(!full, 0)) {
-                            // (the tile reaches over an edge of the first window; the distance is made opaque so that
-                            // none of this is computed ahead of the branch)
-                            int base = 32 * it + 4 * hf - j;         // i - j for register 0
-                            asm volatile("" : "+v"(base));
-#pragma unroll
-                            for (int rr = 0; rr < 16; ++rr) {
-                                const bool ok = (unsigned)(base + 8 * (rr >> 2) + (rr & 3)) < (unsigned)p.w1;
-                                X[rr] = ok ? X[rr] : -INFINITY;
-                            }
-                        }
-                        u32x4 pb[2];
-#pragma unroll
-                        for (int rr = 0; rr < 16; rr += 2)
-                            pb[rr >> 3][(rr & 7) >> 1] = pack_bf16(fast_exp2(X[rr]), fast_exp2(X[rr + 1]));
-                        *reinterpret_cast<u32x4 *>(px + e * 2048) = pb[0];
-                        *reinterpret_cast<u32x4 *>(px + e * 2048 + 1024) = pb[1];
-                        if (e == 0) {
-                            mfma_stream(NProd{}, [&](auto x) { return swz_lane.tr_frag(buf + L::BS, x / DT, x % DT); },
-                                        [&](auto x, const u32x4 &fr) { acc[x % DT] = mfma32(fr, pb[x / DT], acc[x % DT]); });
-                        } else {
-                            pb_late[0] = pb[0];
-                            pb_late[1] = pb[1];
-                        }
-                        __builtin_amdgcn_sched_barrier(0);      // one offset at a time: its fragments are dead before the next one's are loaded
                     }
-                }
-                if (more) build_quarter(nb, (s + 1) & 1, std::true_type{}, 0);
-                __syncthreads();                                // P of the pair is in LDS
+                };
+                u32x4 pb[2], pb_late[2];
+                QB qa;
+                qb_load(qa, nb, nbuf, std::true_type{}, 0);
                 if (on) {
-                    // the S waves now have MFMA and VALU work of their own; this evens out the two halves
-                    const char *buf = pair + L::STEP;
-                    mfma_stream(NProd{}, [&](auto x) { return swz_lane.tr_frag(buf + L::BS, x / DT, x % DT); },
-                                [&](auto x, const u32x4 &fr) { acc[x % DT] = mfma32(fr, pb_late[x / DT], acc[x % DT]); });
+                    f32x16 X0, X1;
+                    start_from(X0, buf0 + L::LSE);
+                    start_from(X1, buf1 + L::LSE);
+                    mfma_stream2(NChain{}, [&](auto kk) { return swz_lane.row_frag(buf0 + L::AS, kk); },
+                                 [&](auto kk, const u32x4 &fr) { X0 = mfma32(fr, k1f[kk], X0); },
+                                 [&](auto x_) { qb_piece(qa, x_, c2); });
+                    qb_store(qa);
+                    edge(X0);
+                    mfma_stream2(NChain{}, [&](auto kk) { return swz_lane.row_frag(buf1 + L::AS, kk); },
+                                 [&](auto kk, const u32x4 &fr) { X1 = mfma32(fr, k1f[kk], X1); },
+                                 [&](auto x_) {
+                                     constexpr int x = decltype(x_)::value;
+                                     pb[x >> 2][x & 3] = pack_bf16(fast_exp2(X0[2 * x]), fast_exp2(X0[2 * x + 1]));
+                                 });
+                    *reinterpret_cast<u32x4 *>(px) = pb[0];
+                    *reinterpret_cast<u32x4 *>(px + 1024) = pb[1];
+                    edge(X1);
+                    mfma_stream2(NProd{}, [&](auto x) { return swz_lane.tr_frag(buf0 + L::BS, x / DT, x % DT); },
+                                 [&](auto x, const u32x4 &fr) { acc[x % DT] = mfma32(fr, pb[x / DT], acc[x % DT]); },
+                                 [&](auto x_) {
+                                     constexpr int x = decltype(x_)::value;
+                                     pb_late[x >> 2][x & 3] = pack_bf16(fast_exp2(X1[2 * x]), fast_exp2(X1[2 * x + 1]));
+                                 });
+                    *reinterpret_cast<u32x4 *>(px + 2048) = pb_late[0];
+                    *reinterpret_cast<u32x4 *>(px + 2048 + 1024) = pb_late[1];
+                } else {
+                    static_for<0, 8>([&](auto x_) { qb_piece(qa, x_, c2); });
+                    qb_store(qa);
                 }
-                if (more) {
-                    build_quarter(nb, (s + 1) & 1, std::false_type{}, 0);
-                    __builtin_amdgcn_sched_barrier(0);
-                    build_quarter(nb, (s + 1) & 1, std::false_type{}, 1);
-                    build_tables(nb, (s + 1) & 1);
-                    next_pair(nb);
+                __syncthreads();                                // P of the pair is in LDS
+                QB qb0, qb1;
+                qb_load(qb0, nb, nbuf, std::false_type{}, 0);
+                qb_load(qb1, nb, nbuf, std::false_type{}, 1);
+                if (on) {
+                    mfma_stream2(NProd{}, [&](auto x) { return swz_lane.tr_frag(buf1 + L::BS, x / DT, x % DT); },
+                                 [&](auto x, const u32x4 &fr) { acc[x % DT] = mfma32(fr, pb_late[x / DT], acc[x % DT]); },
+                                 [&](auto x_) {
+                                     qb_piece(qb0, x_, 1.f);
+                                     qb_piece(qb1, x_, 1.f);
+                                 });
+                } else {
+                    static_for<0, 8>([&](auto x_) {
+                        qb_piece(qb0, x_, 1.f);
+                        qb_piece(qb1, x_, 1.f);
+                    });
                 }
+                qb_store(qb0);
+                qb_store(qb1);
+                build_tables(nb, nbuf);
+                next_pair(nb);
             }
             if (j_ok) store_row<DT>(p.dv1.ptr + b * p.dv1.sb + (int64_t)j * p.dv1.sn + hk * p.dv1.sh + 16 * hf * 2, acc, 1.f);
         } else {
-            // ---- S waves: dP - delta for both offsets, their share of the next pair's tiles; after
-            // the barrier dS = P (dP - delta), dK1^T += A^T dS
+            // ---- S waves: dP - delta for both offsets with a build quarter beside the first chain; after the barrier
+            // dS = P (dP - delta) and dK1^T += A^T dS, the second offset's dS formed beside the first offset's products
             for (int s = 0; s < npairs; ++s) {
                 const bool more = s + 1 < npairs;
                 open_pair(more);
-                const char *pair = lds + (s & 1) * L::PAIR;
+                const char *buf0 = lds + (s & 1) * L::PAIR, *buf1 = buf0 + L::STEP;
+                const int nbuf = (s + 1) & 1;
                 const int it = cur.it;
                 next_pair(cur);
                 const bool on = wave_active && it >= wit_lo && it <= wit_hi;
-                f32x16 dPe[2];
+                f32x16 dP0, dP1;
+                QB qa;
+                qb_load(qa, nb, nbuf, std::true_type{}, 1);
                 if (on) {
-#pragma unroll
-                    for (int e = 0; e < 2; ++e) {
-                        const char *buf = pair + e * L::STEP;
-#pragma unroll
-                        for (int a4 = 0; a4 < 4; ++a4) {
-                            const float4 d4 = *reinterpret_cast<const float4 *>(buf + L::DEL + (8 * a4 + 4 * hf) * 4);
-                            dPe[e][4 * a4] = d4.x;
-                            dPe[e][4 * a4 + 1] = d4.y;
-                            dPe[e][4 * a4 + 2] = d4.z;
-                            dPe[e][4 * a4 + 3] = d4.w;
-                        }
-                        mfma_stream(NChain{}, [&](auto kk) { return swz_lane.row_frag(buf + L::BS, kk); },
-                                    [&](auto kk, const u32x4 &fr) { dPe[e] = mfma32(fr, k1f[kk], dPe[e]); });
-                    }
+                    start_from(dP0, buf0 + L::DEL);
+                    start_from(dP1, buf1 + L::DEL);
+                    mfma_stream2(NChain{}, [&](auto kk) { return swz_lane.row_frag(buf0 + L::BS, kk); },
+                                 [&](auto kk, const u32x4 &fr) { dP0 = mfma32(fr, k1f[kk], dP0); },
+                                 [&](auto x_) { qb_piece(qa, x_, c2); });
+                    qb_store(qa);
+                    mfma_stream(NChain{}, [&](auto kk) { return swz_lane.row_frag(buf1 + L::BS, kk); },
+                                [&](auto kk, const u32x4 &fr) { dP1 = mfma32(fr, k1f[kk], dP1); });
+                } else {
+                    static_for<0, 8>([&](auto x_) { qb_piece(qa, x_, c2); });
+                    qb_store(qa);
                 }
-                // the MFMA chains first, the build after them: measured faster than the other order
-                // (the P waves start the pair with MFMA work as well and then turn to their exponentials)
-                if (more) {
-                    build_quarter(nb, (s + 1) & 1, std::true_type{}, 1);
-                    next_pair(nb);
-                }
+                next_pair(nb);
                 __syncthreads();                                // P of the pair is in LDS
                 if (on) {
+                    u32x4 pq0[2], pq1[2], pb0[2], pb1[2];
 #pragma unroll
-                    for (int e = 0; e < 2; ++e) {
-                        const char *buf = pair + e * L::STEP;
-                        u32x4 pb[2];
-#pragma unroll
-                        for (int hh = 0; hh < 2; ++hh) {
-                            const u32x4 pq = ld_lds16(px + e * 2048 + hh * 1024);
-#pragma unroll
-                            for (int w = 0; w < 4; ++w)
-                                pb[hh][w] = pack_bf16(bf16_lo(pq[w]) * dPe[e][8 * hh + 2 * w], bf16_hi(pq[w]) * dPe[e][8 * hh + 2 * w + 1]);
-                        }
-                        mfma_stream(NProd{}, [&](auto x) { return swz_lane.tr_frag(buf + L::AS, x / DT, x % DT); },
-                                    [&](auto x, const u32x4 &fr) { acc[x % DT] = mfma32(fr, pb[x / DT], acc[x % DT]); });
+                    for (int hh = 0; hh < 2; ++hh) {
+                        pq0[hh] = ld_lds16(px + hh * 1024);
+                        pq1[hh] = ld_lds16(px + 2048 + hh * 1024);
                     }
+#pragma unroll
+                    for (int hh = 0; hh < 2; ++hh)
+#pragma unroll
+                        for (int w = 0; w < 4; ++w)
+                            pb0[hh][w] = pack_bf16(bf16_lo(pq0[hh][w]) * dP0[8 * hh + 2 * w], bf16_hi(pq0[hh][w]) * dP0[8 * hh + 2 * w + 1]);
+                    mfma_stream2(NProd{}, [&](auto x) { return swz_lane.tr_frag(buf0 + L::AS, x / DT, x % DT); },
+                                 [&](auto x, const u32x4 &fr) { acc[x % DT] = mfma32(fr, pb0[x / DT], acc[x % DT]); },
+                                 [&](auto x_) {
+                                     constexpr int x = decltype(x_)::value, hh = x >> 2, w = x & 3;
+                                     pb1[hh][w] = pack_bf16(bf16_lo(pq1[hh][w]) * dP1[8 * hh + 2 * w], bf16_hi(pq1[hh][w]) * dP1[8 * hh + 2 * w + 1]);
+                                 });
+                    mfma_stream(NProd{}, [&](auto x) { return swz_lane.tr_frag(buf1 + L::AS, x / DT, x % DT); },
+                                [&](auto x, const u32x4 &fr) { acc[x % DT] = mfma32(fr, pb1[x / DT], acc[x % DT]); });
                 }
             }
             if (j_ok) store_row<DT>(p.dk1.ptr + b * p.dk1.sb + (int64_t)j * p.dk1.sn + hk * p.dk1.sh + 16 * hf * 2, acc, kLn2);   // A carried scale log2(e)
