@@ -223,3 +223,29 @@ def test_reference_import_paths_resolve_to_this_build():
     assert HOA is HigherOrderAttention is S.HigherOrderAttention and TwoSimplicialMHA is S.TwoSimplicialMHA
     attn = SlidingWindowTwoSimplicialMHA(dim=512, dim_head=64, heads=8)
     assert isinstance(attn, HigherOrderAttention) and TwoSimplicialTransformer is not None
+
+
+def test_saved_partials_budget_is_global_per_device(monkeypatch):
+    """The forward keeps its per-offset partials only within a per-call cap, a per-device total and
+    half of the memory still available; buffers that die give their bytes back."""
+    from simplicial_attention_amd.two_simplicial_attention import _PartialsBudget
+    monkeypatch.delenv('SA2_SAVE_PARTIALS_MAX_GIB', raising=False)
+    monkeypatch.delenv('SA2_SAVE_PARTIALS_TOTAL_FRACTION', raising=False)
+    gib = 1 << 30
+    budget = _PartialsBudget()
+    info = (200 * gib, 288 * gib)                       # (available, total)
+    assert not budget.admit(0, 'cuda:0', info)
+    assert not budget.admit(17 * gib, 'cuda:0', info)   # per-call cap (16 GiB)
+    for _ in range(4):
+        assert budget.admit(16 * gib, 'cuda:0', info)   # 64 GiB alive
+    assert budget.admit(8 * gib, 'cuda:0', info)        # 72 GiB = a quarter of the device
+    assert not budget.admit(1 * gib, 'cuda:0', info)    # the total is spent ...
+    assert budget.admit(1 * gib, 'cuda:1', info)        # ... on that device only
+    budget.release(16 * gib, 0)
+    assert budget.admit(16 * gib, 'cuda:0', info)
+    assert not _PartialsBudget().admit(3 * gib, 'cuda:0', (4 * gib, 288 * gib))   # more than half of what is left
+    monkeypatch.setenv('SA2_SAVE_PARTIALS_MAX_GIB', '0')
+    assert not _PartialsBudget().admit(1, 'cuda:0', info)
+    monkeypatch.setenv('SA2_SAVE_PARTIALS_MAX_GIB', '16')
+    monkeypatch.setenv('SA2_SAVE_PARTIALS_TOTAL_FRACTION', '0.01')
+    assert not _PartialsBudget().admit(3 * gib, 'cuda:0', info)
