@@ -56,7 +56,7 @@ typedef struct sa2_problem {
     int32_t seq_len;
     int32_t heads;      /* query heads */
     int32_t kv_heads;   /* key/value heads, divides heads */
-    int32_t dim_head;   /* 64 or 128 */
+    int32_t dim_head;   /* 32, 64 or 128 */
     int32_t w1;         /* window of the first key/value set  (reference default 512) */
     int32_t w2;         /* window of the second key/value set (reference default 32), any value >= 1 */
     int32_t causal;     /* must be 1 */
@@ -94,7 +94,7 @@ int sa2_version(void);
 /* Message of the last failing call on this thread ("" if none). */
 const char *sa2_last_error(void);
 
-/* 1 if the kernels cover this configuration (dim_head 64 or 128, any w1 >= 1 and w2 >= 1, bf16),
+/* 1 if the kernels cover this configuration (dim_head 32, 64 or 128, any w1 >= 1 and w2 >= 1, bf16),
  * else 0.  Replaces the silent limits of the reference (HEAD_DIM fixed to 64, w2 <= 32:
  * triton_two_simplicial_attention.py:51,291,508,586). */
 int sa2_supported(int32_t dim_head, int32_t w1, int32_t w2, int32_t dtype);

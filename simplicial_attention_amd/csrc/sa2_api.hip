@@ -41,8 +41,8 @@ int check_problem(const sa2_problem *p) {
     if (p->w1 < 1 || p->w2 < 1) return fail(SA2_ERR_BAD_SHAPE, "windows w1=%d w2=%d must be >= 1", p->w1, p->w2);
     if (p->causal != 1) return fail(SA2_ERR_UNSUPPORTED, "only causal=1 is defined for the sliding windows");
     if (p->dtype != SA2_BF16) return fail(SA2_ERR_UNSUPPORTED, "dtype %d is not supported (bf16 only)", p->dtype);
-    if (p->dim_head != 64 && p->dim_head != 128)
-        return fail(SA2_ERR_UNSUPPORTED, "dim_head=%d is not supported (64 or 128)", p->dim_head);
+    if (p->dim_head != 32 && p->dim_head != 64 && p->dim_head != 128)
+        return fail(SA2_ERR_UNSUPPORTED, "dim_head=%d is not supported (32, 64 or 128)", p->dim_head);
     if (!(p->scale > 0.f) || !std::isfinite(p->scale)) return fail(SA2_ERR_BAD_SHAPE, "scale must be positive and finite");
     if ((int64_t)p->batch * p->heads * ((p->seq_len + 31) / 32) > 0x7fffffffll)
         return fail(SA2_ERR_BAD_SHAPE, "problem too large for a 1-D grid");
@@ -93,6 +93,21 @@ int after_launch(const char *what) {
         if (rc_ != SA2_OK) return rc_; \
     } while (0)
 
+// Runs `stmt` with the compile-time constant DH set to the problem's head dimension (validated by check_problem).
+#define SA2_FOR_DIM_HEAD(dim_head, stmt)        \
+    do {                                        \
+        if ((dim_head) == 128) {                \
+            constexpr int DH = 128;             \
+            stmt;                               \
+        } else if ((dim_head) == 64) {          \
+            constexpr int DH = 64;              \
+            stmt;                               \
+        } else {                                \
+            constexpr int DH = 32;              \
+            stmt;                               \
+        }                                       \
+    } while (0)
+
 // Scratch of sa2_bwd_noalloc: delta rows followed by the dK2/dV2 partial rows.  A file-scope device
 // array: every GPU the library runs on holds its own copy, at its own address, until the process
 // ends.  In host code the array's name is only a handle for hipGetSymbolAddress; kernels and
@@ -130,7 +145,7 @@ int sa2_version(void) { return SA2_VERSION; }
 const char *sa2_last_error(void) { return g_err; }
 
 int sa2_supported(int32_t dim_head, int32_t w1, int32_t w2, int32_t dtype) {
-    return (dim_head == 64 || dim_head == 128) && w1 >= 1 && w2 >= 1 && dtype == SA2_BF16;
+    return (dim_head == 32 || dim_head == 64 || dim_head == 128) && w1 >= 1 && w2 >= 1 && dtype == SA2_BF16;
 }
 
 static int check_saved(const sa2_saved *saved) {
@@ -179,9 +194,8 @@ int sa2_fwd(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, 
     const int grid = prob->batch * prob->heads * ((prob->seq_len + 31) / 32);
     // dim_head 64 with a second window of up to 32: the instance that fits four waves per SIMD
     // (two workgroups per CU); everything else: the general kernel (any second window)
-    if (prob->dim_head == 128) hipLaunchKernelGGL(sa2::fwd_kernel<128>, dim3(grid), dim3(512), 0, s, k);
-    else if (prob->w2 <= 32) hipLaunchKernelGGL((sa2::fwd8_kernel<64, 32>), dim3(grid), dim3(512), 0, s, k);
-    else hipLaunchKernelGGL(sa2::fwd_kernel<64>, dim3(grid), dim3(512), 0, s, k);
+    if (prob->dim_head == 64 && prob->w2 <= 32) hipLaunchKernelGGL((sa2::fwd8_kernel<64, 32>), dim3(grid), dim3(512), 0, s, k);
+    else SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL(sa2::fwd_kernel<DH>, dim3(grid), dim3(512), 0, s, k));
     return after_launch("forward");
 }
 
@@ -202,10 +216,7 @@ int sa2_bwd_delta(const sa2_problem *prob, const sa2_tensor *out, const sa2_tens
     int lanes_per_row = prob->dim_head / 8;
     int rows_per_block = 256 / lanes_per_row;
     int grid = (int)((rows + rows_per_block - 1) / rows_per_block);
-    if (prob->dim_head == 128)
-        hipLaunchKernelGGL(sa2::delta_kernel<128>, dim3(grid), dim3(256), 0, s, k);
-    else
-        hipLaunchKernelGGL(sa2::delta_kernel<64>, dim3(grid), dim3(256), 0, s, k);
+    SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL(sa2::delta_kernel<DH>, dim3(grid), dim3(256), 0, s, k));
     return after_launch("delta");
 }
 
@@ -286,32 +297,22 @@ int sa2_bwd_dq_dkv2(const sa2_problem *prob, const sa2_tensor *q, const sa2_tens
         k.t_save = static_cast<char *>(saved->t);
         k.m_save = saved->m;
     }
-    if (prob->dim_head == 128) {
-        hipLaunchKernelGGL((sa2::bwd_q_kernel<128, true>), dim3(grid), dim3(512), 0, s, k, ws, halo);
-        if (pass != 1 && !use_saved) hipLaunchKernelGGL((sa2::bwd_q_kernel<128, false>), dim3(grid), dim3(512), 0, s, k, ws, halo);
-    } else {
-        hipLaunchKernelGGL((sa2::bwd_q_kernel<64, true>), dim3(grid), dim3(512), 0, s, k, ws, halo);
-        if (pass != 1 && !use_saved) hipLaunchKernelGGL((sa2::bwd_q_kernel<64, false>), dim3(grid), dim3(512), 0, s, k, ws, halo);
-    }
+    SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL((sa2::bwd_q_kernel<DH, true>), dim3(grid), dim3(512), 0, s, k, ws, halo));
+    if (pass != 1 && !use_saved)
+        SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL((sa2::bwd_q_kernel<DH, false>), dim3(grid), dim3(512), 0, s, k, ws, halo));
     SA2_TRY(after_launch("dq/dk2/dv2"));
     if (pass == 1) return SA2_OK;    // profiling build, one pass: leave the reductions out of its timing
     if (use_saved) {
         const int rpb = 256 / (prob->dim_head / 8);
         const int dgrid = prob->batch * prob->kv_heads * ((prob->seq_len + rpb - 1) / rpb);
-        if (prob->dim_head == 128)
-            hipLaunchKernelGGL(sa2::dv2_from_saved_kernel<128>, dim3(dgrid), dim3(256), 0, s, k);
-        else
-            hipLaunchKernelGGL(sa2::dv2_from_saved_kernel<64>, dim3(dgrid), dim3(256), 0, s, k);
+        SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL(sa2::dv2_from_saved_kernel<DH>, dim3(dgrid), dim3(256), 0, s, k));
         SA2_TRY(after_launch("dv2 from saved partials"));
     }
     const int64_t rows = (int64_t)prob->batch * prob->kv_heads * prob->seq_len;
     const int rows_per_block = 256 / (prob->dim_head / 8);
     const int cgrid = (int)((rows + rows_per_block - 1) / rows_per_block);
     const int with_dv2 = use_saved ? 0 : 1;
-    if (prob->dim_head == 128)
-        hipLaunchKernelGGL(sa2::dk2_dv2_combine_kernel<128>, dim3(cgrid), dim3(256), 0, s, k, ws, 32 + halo, with_dv2);
-    else
-        hipLaunchKernelGGL(sa2::dk2_dv2_combine_kernel<64>, dim3(cgrid), dim3(256), 0, s, k, ws, 32 + halo, with_dv2);
+    SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL(sa2::dk2_dv2_combine_kernel<DH>, dim3(cgrid), dim3(256), 0, s, k, ws, 32 + halo, with_dv2));
     return after_launch("dk2/dv2 combine");
 }
 
@@ -326,11 +327,13 @@ int sa2_bwd_dkv1(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor 
     k.dv1 = dev(dv1);
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
     int grid = prob->batch * prob->kv_heads * ((prob->seq_len + 127) / 128);
-    // dim_head 128: the two waves of a slab split the contractions; dim_head 64: each wave forms both outputs
+    // dim_head 128: the two waves of a slab split the contractions; dim_head 64 and 32: each wave forms both outputs
     if (prob->dim_head == 128)
         hipLaunchKernelGGL((sa2::bwd_kv8_kernel<128, sa2::kKvSplit>), dim3(grid), dim3(512), 0, s, k);
-    else
+    else if (prob->dim_head == 64)
         hipLaunchKernelGGL((sa2::bwd_kv8_kernel<64, sa2::kKvBoth>), dim3(grid), dim3(512), 0, s, k);
+    else
+        hipLaunchKernelGGL((sa2::bwd_kv8_kernel<32, sa2::kKvBoth>), dim3(grid), dim3(512), 0, s, k);
     return after_launch("dk1/dv1");
 }
 
@@ -422,10 +425,7 @@ int sa2_qkv_norm_fwd(const sa2_problem *prob, const void *qkv, int64_t row_strid
     np.eps = eps;
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
     const int grid = norm_groups(prob);
-    if (prob->dim_head == 128)
-        hipLaunchKernelGGL(sa2::qkv_norm_fwd_kernel<128>, dim3(grid), dim3(256), 0, s, np);
-    else
-        hipLaunchKernelGGL(sa2::qkv_norm_fwd_kernel<64>, dim3(grid), dim3(256), 0, s, np);
+    SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL(sa2::qkv_norm_fwd_kernel<DH>, dim3(grid), dim3(256), 0, s, np));
     return after_launch("qkv norm forward");
 }
 
@@ -455,10 +455,7 @@ int sa2_qkv_norm_bwd(const sa2_problem *prob, const void *qkv, int64_t row_strid
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
     const int groups = norm_groups(prob);
     const int blocks = groups < kNormMaxBlocks ? groups : kNormMaxBlocks;
-    if (prob->dim_head == 128)
-        hipLaunchKernelGGL(sa2::qkv_norm_bwd_kernel<128>, dim3(blocks), dim3(256), 0, s, np, groups);
-    else
-        hipLaunchKernelGGL(sa2::qkv_norm_bwd_kernel<64>, dim3(blocks), dim3(256), 0, s, np, groups);
+    SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL(sa2::qkv_norm_bwd_kernel<DH>, dim3(blocks), dim3(256), 0, s, np, groups));
     SA2_TRY(after_launch("qkv norm backward"));
     const int n = 5 * prob->dim_head;
     hipLaunchKernelGGL(sa2::qkv_norm_dw_kernel, dim3((n + 15) / 16), dim3(256), 0, s, np.dw_part, dw, blocks, n);

@@ -89,7 +89,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     constexpr int KS = D / 16, DT = D / 32, PPR = D / 8;
     using L = Kv8Cfg<D, MODE>;
     constexpr bool DK = L::DK, TWO = MODE == kKvBoth, SPLIT = MODE == kKvSplit;
-    static_assert(!TWO || D == 64, "both accumulators fit two waves per SIMD at D = 64 only");
+    static_assert(!TWO || D <= 64, "both accumulators fit two waves per SIMD up to D = 64 only");
     constexpr int PITCH = L::PITCH;
     __shared__ __attribute__((aligned(16))) char lds[L::LDS];
 
@@ -297,7 +297,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                 product(xv, L::K2S, std::true_type{});
             }
             if constexpr (BOTH) __builtin_amdgcn_sched_barrier(0);   // one product at a time: the dk1 pass has no registers for both
-            if (BOTH || tid >= PIECES) {
+            if (BOTH || (tid >= PIECES && tid < 2 * PIECES)) {
                 unpack(L::DOS, 1.f);
                 product(xv, L::V2S, std::false_type{});
             }
@@ -346,7 +346,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
         constexpr int NF = decltype(n_tag)::value;
         constexpr int W = 3;
         u32x4 f[W];
-        static_for<0, W>([&](auto s_) { f[s_] = frag(s_); });
+        static_for<0, (W < NF ? W : NF)>([&](auto s_) { f[s_] = frag(s_); });
         __builtin_amdgcn_sched_barrier(0);
         static_for<0, NF>([&](auto s_) {
             constexpr int x = decltype(s_)::value;

@@ -62,30 +62,6 @@ __host__ __device__ inline int64_t qk2_ws_floats(int B, int H, int N, int D, int
     return 2ll * B * H * ((N + 31) / 32) * srows * D;
 }
 
-template <int NS, typename F>
-__device__ __forceinline__ void with_slice(int s, F &&f) {
-    static_assert(NS == 4 || NS == 8, "slice count");
-    if constexpr (NS == 8) {
-        switch (s & 7) {
-            case 0: f(std::integral_constant<int, 0>{}); break;
-            case 1: f(std::integral_constant<int, 1>{}); break;
-            case 2: f(std::integral_constant<int, 2>{}); break;
-            case 3: f(std::integral_constant<int, 3>{}); break;
-            case 4: f(std::integral_constant<int, 4>{}); break;
-            case 5: f(std::integral_constant<int, 5>{}); break;
-            case 6: f(std::integral_constant<int, 6>{}); break;
-            default: f(std::integral_constant<int, 7>{}); break;
-        }
-    } else {
-        switch (s & 3) {
-            case 0: f(std::integral_constant<int, 0>{}); break;
-            case 1: f(std::integral_constant<int, 1>{}); break;
-            case 2: f(std::integral_constant<int, 2>{}); break;
-            default: f(std::integral_constant<int, 3>{}); break;
-        }
-    }
-}
-
 template <int D, bool DQ>
 __global__ __launch_bounds__(512) void bwd_q_kernel(KParams p, float *ws, int halo) {
     using C = QCfg<D, DQ>;
@@ -301,14 +277,14 @@ __global__ __launch_bounds__(512) void bwd_q_kernel(KParams p, float *ws, int ha
                     else return RT::tr_frag(tb, (s - NROW) / DT, (s - NROW) % DT);
                 };
                 u32x4 f[W];
-                static_for<0, W>([&](auto s) { f[s] = fragment(s); });
+                static_for<0, (W < NFR ? W : NFR)>([&](auto s) { f[s] = fragment(s); });
                 f32x16 dP = neg_delta;      // DQ: the chain starts from -delta_i, so dP - delta costs no VALU work
                 __builtin_amdgcn_sched_barrier(0);
                 static_for<0, NROW>([&](auto sc_) {
                     constexpr int s = decltype(sc_)::value;
                     if constexpr (s < KS) X = mfma32(f[s % W], A[s], X);
                     else dP = mfma32(f[s % W], Bv[DQ ? s - KS : 0], dP);
-                    f[s % W] = fragment(std::integral_constant<int, s + W>{});
+                    if constexpr (s + W < NFR) f[s % W] = fragment(std::integral_constant<int, s + W>{});
                     __builtin_amdgcn_sched_barrier(0);
                 });
                 // weights of the first 16 tile rows, their products, the weights of the other 16 rows between them
@@ -379,8 +355,9 @@ __global__ __launch_bounds__(512) void bwd_q_kernel(KParams p, float *ws, int ha
                 }
             };
             for (int ph = 0; ph < 8; ++ph) {
-                // D = 128: eight slices.  D = 64: four slices; waves 0-3 use phases 0-3, waves 4-7 phases 4-7
-                if (DT == 4 || (ph >> 2) == (wave >> 2)) with_slice<2 * DT>(wave + ph, add_slice);
+                // 2 DT slices: the waves form 8 / (2 DT) groups that take turns, group g owns the phases 2 DT g ..
+                // 2 DT g + 2 DT - 1 (D = 128: one group, every wave works in every phase)
+                if (DT == 4 || ph / (2 * DT) == wave / (2 * DT)) with_slice<2 * DT>(wave + ph, add_slice);
                 if (ph == 7 && r + 1 < R) write_rows(r);    // (their slots are not in use in this round)
                 __syncthreads();
             }
@@ -399,15 +376,20 @@ __global__ __launch_bounds__(512) void bwd_q_kernel(KParams p, float *ws, int ha
         if (ir < N) {
             const float *src = dqs + row * C::SPITCH + seg * SEG;
             char *orow = p.dq.ptr + b * p.dq.sb + (int64_t)ir * p.dq.sn + h * p.dq.sh + seg * SEG * 2;
-            float4 a = *reinterpret_cast<const float4 *>(src);
             if constexpr (SEG == 8) {
+                float4 a = *reinterpret_cast<const float4 *>(src);
                 float4 bq = *reinterpret_cast<const float4 *>(src + 4);
                 u32x4 ov = {pack_bf16(a.x * p.scale, a.y * p.scale), pack_bf16(a.z * p.scale, a.w * p.scale),
                             pack_bf16(bq.x * p.scale, bq.y * p.scale), pack_bf16(bq.z * p.scale, bq.w * p.scale)};
                 st_global16(orow, ov);
-            } else {
+            } else if constexpr (SEG == 4) {
+                float4 a = *reinterpret_cast<const float4 *>(src);
                 u32x2 ov = {pack_bf16(a.x * p.scale, a.y * p.scale), pack_bf16(a.z * p.scale, a.w * p.scale)};
                 *reinterpret_cast<u32x2 *>(orow) = ov;
+            } else {
+                static_assert(SEG == 2, "head dimension 32, 64 or 128");
+                float2 a = *reinterpret_cast<const float2 *>(src);
+                *reinterpret_cast<uint32_t *>(orow) = pack_bf16(a.x * p.scale, a.y * p.scale);
             }
         }
     }

@@ -151,6 +151,34 @@ __device__ __forceinline__ void store_row(char *orow, const f32x16 (&acc)[DT], f
     }
 }
 
+// f(integral_constant<int, s mod NS>) for a run-time s (NS = 2, 4 or 8)
+template <int NS, typename F>
+__device__ __forceinline__ void with_slice(int s, F &&f) {
+    static_assert(NS == 2 || NS == 4 || NS == 8, "slice count");
+    if constexpr (NS == 8) {
+        switch (s & 7) {
+            case 0: f(std::integral_constant<int, 0>{}); break;
+            case 1: f(std::integral_constant<int, 1>{}); break;
+            case 2: f(std::integral_constant<int, 2>{}); break;
+            case 3: f(std::integral_constant<int, 3>{}); break;
+            case 4: f(std::integral_constant<int, 4>{}); break;
+            case 5: f(std::integral_constant<int, 5>{}); break;
+            case 6: f(std::integral_constant<int, 6>{}); break;
+            default: f(std::integral_constant<int, 7>{}); break;
+        }
+    } else if constexpr (NS == 4) {
+        switch (s & 3) {
+            case 0: f(std::integral_constant<int, 0>{}); break;
+            case 1: f(std::integral_constant<int, 1>{}); break;
+            case 2: f(std::integral_constant<int, 2>{}); break;
+            default: f(std::integral_constant<int, 3>{}); break;
+        }
+    } else {
+        if (s & 1) f(std::integral_constant<int, 1>{});
+        else f(std::integral_constant<int, 0>{});
+    }
+}
+
 // Grid index -> logical work item such that the eight XCDs (which receive
 // consecutive workgroup ids round-robin) each walk a contiguous range of items.
 __device__ __forceinline__ int xcd_contiguous(int wg, int total) {

@@ -459,29 +459,11 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
                 *reinterpret_cast<float4 *>(dst) = a0;
                 *reinterpret_cast<float4 *>(dst + 4) = a1;
             };
+            // 2 DT slices of eight registers: the waves form 8 / (2 DT) groups that take turns, group g owns the
+            // phases 2 DT g .. 2 DT g + 2 DT - 1 and its wave w the slice (w + ph) mod 2 DT in phase ph
             for (int ph = 0; ph < 8; ++ph) {
-                if constexpr (DT == 4) {
-                    switch ((wave + ph) & 7) {
-                        case 0: add_slice(std::integral_constant<int, 0>{}, ph == 0); break;
-                        case 1: add_slice(std::integral_constant<int, 1>{}, ph == 0); break;
-                        case 2: add_slice(std::integral_constant<int, 2>{}, ph == 0); break;
-                        case 3: add_slice(std::integral_constant<int, 3>{}, ph == 0); break;
-                        case 4: add_slice(std::integral_constant<int, 4>{}, ph == 0); break;
-                        case 5: add_slice(std::integral_constant<int, 5>{}, ph == 0); break;
-                        case 6: add_slice(std::integral_constant<int, 6>{}, ph == 0); break;
-                        default: add_slice(std::integral_constant<int, 7>{}, ph == 0); break;
-                    }
-                } else {
-                    // D = 64: four slices; waves 0-3 use phases 0-3, waves 4-7 phases 4-7
-                    if ((ph >> 2) == (wave >> 2)) {
-                        switch ((wave + ph) & 3) {
-                            case 0: add_slice(std::integral_constant<int, 0>{}, ph == 0); break;
-                            case 1: add_slice(std::integral_constant<int, 1>{}, ph == 0); break;
-                            case 2: add_slice(std::integral_constant<int, 2>{}, ph == 0); break;
-                            default: add_slice(std::integral_constant<int, 3>{}, ph == 0); break;
-                        }
-                    }
-                }
+                constexpr int NS = 2 * DT;
+                if (NS == 8 || ph / NS == wave / NS) with_slice<NS>(wave + ph, [&](auto tag) { add_slice(tag, ph % NS == 0 && (NS == 8 || wave / NS == 0)); });
                 if (ph == 7 && r + 1 < R) write_rows(r);    // (their slots are not in use in this round)
                 __syncthreads();
             }
@@ -512,12 +494,10 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
         char *rrow = p.o_lo.ptr ? p.o_lo.ptr + b * p.o_lo.sb + (int64_t)ir * p.o_lo.sn + h * p.o_lo.sh + seg * SEG * 2 : nullptr;
         float o[SEG];
 #pragma unroll
-        for (int x = 0; x < SEG; x += 4) {
-            float4 v = *reinterpret_cast<const float4 *>(src + x);
+        for (int x = 0; x < SEG; x += 2) {
+            float2 v = *reinterpret_cast<const float2 *>(src + x);
             o[x] = v.x * inv;
             o[x + 1] = v.y * inv;
-            o[x + 2] = v.z * inv;
-            o[x + 3] = v.w * inv;
         }
         if constexpr (SEG == 8) {
             u32x4 ov, rv;
@@ -528,7 +508,7 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
             }
             st_global16(orow, ov);
             if (rrow) st_global16(rrow, rv);
-        } else {
+        } else if constexpr (SEG == 4) {
             u32x2 ov, rv;
 #pragma unroll
             for (int w = 0; w < 2; ++w) {
@@ -537,6 +517,11 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
             }
             *reinterpret_cast<u32x2 *>(orow) = ov;
             if (rrow) *reinterpret_cast<u32x2 *>(rrow) = rv;
+        } else {
+            static_assert(SEG == 2, "head dimension 32, 64 or 128");
+            const uint32_t ov = pack_bf16(o[0], o[1]);
+            *reinterpret_cast<uint32_t *>(orow) = ov;
+            if (rrow) *reinterpret_cast<uint32_t *>(rrow) = pack_bf16(o[0] - bf16_lo(ov), o[1] - bf16_hi(ov));
         }
         if (seg == 0) p.lse[((int64_t)b * p.H + h) * N + ir] = (xm[row] + __builtin_amdgcn_logf(L)) * kLn2;
     }

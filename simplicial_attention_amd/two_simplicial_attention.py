@@ -130,7 +130,7 @@ class SlidingTwoSimplicialAttention(Function):
             raise ValueError('window sizes must be at least 1')
         lib = _native.load()
         if not lib.sa2_supported(dim, w1, w2, _native.SA2_BF16):
-            raise NotImplementedError(f'dim_head={dim}, w1={w1}, w2={w2} is not covered by the kernels (dim_head 64 or 128)')
+            raise NotImplementedError(f'dim_head={dim}, w1={w1}, w2={w2} is not covered by the kernels (dim_head 32, 64 or 128)')
 
         q, k1, k2, v1, v2 = (_unit_inner_stride(t) for t in tensors)
         scale = dim ** -0.5 if scale is None else float(scale)
@@ -208,7 +208,7 @@ def sliding_two_simplicial_attn(
     Beyond the reference (whose kernels are written for bf16 and a head dimension of
     64): float16 and float32 tensors are computed in bfloat16 and the result returned
     in the input dtype; any head dimension up to 128, and a value head dimension
-    different from the query/key one, are zero-padded to the kernels' 64 or 128
+    different from the query/key one, are zero-padded to the kernels' 32, 64 or 128
     (padded query/key channels add nothing to the logits, padded value channels give
     zero outputs that are sliced off; the softmax scale stays that of the true
     query/key dimension).
@@ -226,9 +226,9 @@ def sliding_two_simplicial_attn(
     dim = max(dim_qk, dim_v)
     if dim > 128:
         raise NotImplementedError(f'head dimension {dim} is not covered by the kernels (at most 128)')
-    if dtype is torch.bfloat16 and dim_qk == dim_v and dim in (64, 128):
+    if dtype is torch.bfloat16 and dim_qk == dim_v and dim in (32, 64, 128):
         return _sliding_two_simplicial_attn(q, k1, k2, v1, v2, w1, w2, causal)
-    dim_kernel = 64 if dim <= 64 else 128
+    dim_kernel = 32 if dim <= 32 else (64 if dim <= 64 else 128)
 
     def prepare(t):
         t = t.to(torch.bfloat16)

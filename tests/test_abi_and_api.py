@@ -41,7 +41,9 @@ def test_supported_matrix(lib):
     assert lib.sa2_supported(128, 512, 64, 0) == 1
     assert lib.sa2_supported(128, 512, 65, 0) == 1
     assert lib.sa2_supported(64, 8192, 8192, 0) == 1
-    assert lib.sa2_supported(32, 512, 32, 0) == 0
+    assert lib.sa2_supported(32, 512, 32, 0) == 1
+    assert lib.sa2_supported(96, 512, 32, 0) == 0
+    assert lib.sa2_supported(256, 512, 32, 0) == 0
     assert lib.sa2_supported(128, 0, 32, 0) == 0
     assert lib.sa2_supported(128, 512, 32, 1) == 0
 

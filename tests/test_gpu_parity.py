@@ -28,6 +28,10 @@ CASES = [
     (1, 1, 1, 1, 128, 512, 32),       # a single row
     (1, 17, 2, 1, 64, 512, 32),       # less than one tile
     (2, 31, 4, 2, 128, 8, 32),        # less than one tile, second window wider than the sequence
+    (1, 128, 4, 4, 32, 128, 128),     # head dimension 32 (native instance): shape of the reference's CPU-runnable case
+    (2, 333, 4, 2, 32, 100, 32),      # head dimension 32, ragged N, grouped heads
+    (1, 200, 2, 1, 32, 48, 70),       # head dimension 32, several offset blocks
+    (1, 19, 2, 2, 32, 512, 32),       # head dimension 32, less than one tile
 ]
 
 
@@ -46,7 +50,7 @@ def _random_shapes(count, seed=1234):
     rng = random.Random(seed)
     shapes = []
     for _ in range(count):
-        d = rng.choice([64, 128])
+        d = rng.choice([32, 64, 128])
         hk = rng.choice([1, 2])
         hq = hk * rng.choice([1, 2])
         n = rng.choice([rng.randint(1, 40), rng.randint(33, 130), rng.randint(131, 420)])
@@ -142,7 +146,7 @@ def test_lse_matches_oracle():
     assert torch.allclose(lse.cpu(), ref, atol=2e-2, rtol=1e-2)
 
 
-@pytest.mark.parametrize('shape', [(2, 320, 4, 2, 128, 96, 16), (1, 200, 2, 2, 64, 64, 32)])
+@pytest.mark.parametrize('shape', [(2, 320, 4, 2, 128, 96, 16), (1, 200, 2, 2, 64, 64, 32), (1, 200, 2, 1, 32, 64, 32)])
 def test_backward_that_recomputes_instead_of_using_saved_partials(shape, monkeypatch):
     """SA2_SAVE_PARTIALS_MAX_GIB=0: the forward keeps no per-offset T and dV2 comes from
     the recomputing pass (what the reference does)."""
@@ -161,7 +165,7 @@ def test_backward_that_recomputes_instead_of_using_saved_partials(shape, monkeyp
     (torch.bfloat16, 96, 96, 100, 512, 32),
 ])
 def test_other_head_dimensions_and_dtypes(dtype, dqk, dv, n, w1, w2):
-    """Head dimensions other than 64/128, a value head dimension of its own, and float16 /
+    """Head dimensions other than 32/64/128 (and the native 32), a value head dimension of its own, and float16 /
     float32 tensors: the functional wrapper pads and casts around the bf16 kernels; output
     and gradients come back in the caller's dtype and shapes.  The oracle works on the
     bf16-rounded values with the scale of the true query/key dimension."""
