@@ -265,14 +265,15 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
         // The fragment reads of a step sit between its MFMAs, a scheduling fence behind every MFMA and its reads
         // keeps them there: the V1 fragments of the tile along its logit chain, the K1 fragments of the next tile
         // along the value chain.
-        auto value_products = [&](const u32x4 (&pb)[2], bool next_kf) {
+        // (the K1 fragments behind the round's last tile are those of the next round's first tile: the ring runs on)
+        auto value_products = [&](const u32x4 (&pb)[2]) {
             const char *kbase = lds + b_nxt + k_lane;
 #pragma unroll
             for (int m = 0; m < 2 * DT; ++m) {
                 const int k2s = m / DT, dt = m % DT;
                 u32x4 v = {vf[dt][k2s][0][0], vf[dt][k2s][0][1], vf[dt][k2s][1][0], vf[dt][k2s][1][1]};
                 T[dt] = mfma32(v, pb[k2s], T[dt]);
-                if (next_kf) kf[m] = ld_lds16(kbase + C::RT::row_imm(m));
+                kf[m] = ld_lds16(kbase + C::RT::row_imm(m));
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
@@ -344,7 +345,7 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
                 }
                 u32x4 pb[2];
                 exponentials(X, pb);
-                value_products(pb, 1 < NT);
+                value_products(pb);
                 close_step();
                 n = 1;
             }
@@ -389,7 +390,7 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
                     NMv = splat16(nm);
                     exponentials(X, pb);
                 }
-                value_products(pb, n + 1 < NT);
+                value_products(pb);
                 close_step();
             }
         }
