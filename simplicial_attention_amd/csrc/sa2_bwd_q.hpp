@@ -46,8 +46,9 @@ struct QCfg {
     static constexpr int SPITCH = D + 4;              // floats per row of the fp32 rows
     static constexpr int DQS = RING;                  // dq rows [32][SPITCH]            (DQ only)
     static constexpr int SC = RING + (DQ ? 32 * SPITCH * 4 : 0);   // scatter rows, circular [64][SPITCH]
-    static constexpr int QS = SC + 64 * SPITCH * 4;                // q rows   [32][PITCH]
-    static constexpr int DOS = QS + TILE;                          // do rows  [32][PITCH]
+    static constexpr int QS = SC + 64 * SPITCH * 4;                // q rows times scale log2(e), fp32 [32][QPITCH bytes]
+    static constexpr int QPITCH = D * 4 + 16;
+    static constexpr int DOS = QS + 32 * QPITCH;                   // do rows  [32][PITCH]
     static constexpr int K2S = DOS + TILE;                         // k2 rows, circular [64][PITCH]
     static constexpr int V2S = K2S + 64 * PITCH;                   // v2 rows, circular [64][PITCH]  (DQ only)
     static constexpr int MASKS = DQ ? V2S + 64 * PITCH : V2S;      // additive masks, 3 tables [4 quarters][64 lanes][4 floats]
@@ -143,7 +144,12 @@ __global__ __launch_bounds__(512) void bwd_q_kernel(KParams p, float *ws, int ha
             const int row = x / PPR, col = (x % PPR) * 16;
             int ii = i0 + row;
             ii = ii < N ? ii : N - 1;
-            *reinterpret_cast<u32x4 *>(lds + C::QS + row * PITCH + col) = ld_global16(qg + (int64_t)ii * p.q.sn + col);
+            // q unpacked and scaled once per workgroup (the operand build of every offset and the dK2 rows multiply by it)
+            const u32x4 fq = ld_global16(qg + (int64_t)ii * p.q.sn + col);
+            const float c2 = p.scale_log2e;
+            float4 *qdst = reinterpret_cast<float4 *>(lds + C::QS + row * C::QPITCH + col * 2);
+            qdst[0] = make_float4(bf16_lo(fq[0]) * c2, bf16_hi(fq[0]) * c2, bf16_lo(fq[1]) * c2, bf16_hi(fq[1]) * c2);
+            qdst[1] = make_float4(bf16_lo(fq[2]) * c2, bf16_hi(fq[2]) * c2, bf16_lo(fq[3]) * c2, bf16_hi(fq[3]) * c2);
             *reinterpret_cast<u32x4 *>(lds + C::DOS + row * PITCH + col) = ld_global16(dog + (int64_t)ii * p.dout.sn + col);
         }
         for (int x = tid; x < 39 * PPR; x += 512) {
@@ -222,15 +228,16 @@ __global__ __launch_bounds__(512) void bwd_q_kernel(KParams p, float *ws, int ha
         const bool wave_on = wave_any(col_ok);
         const int slot = (c - dlt) & 63;              // slot of row k = i - dlt in the circular rows
         {
-            const char *qr = lds + C::QS + c * PITCH + 16 * hf;
+            const char *qr = lds + C::QS + c * C::QPITCH + 32 * hf;
             const char *k2r = lds + C::K2S + slot * PITCH + 16 * hf;
-            const float c2 = p.scale_log2e;
 #pragma unroll
             for (int kk = 0; kk < KS; ++kk) {
-                const u32x4 fq = ld_lds16(qr + 32 * kk), fk = ld_lds16(k2r + 32 * kk);
-#pragma unroll
-                for (int w = 0; w < 4; ++w)
-                    A[kk][w] = pack_bf16(bf16_lo(fq[w]) * bf16_lo(fk[w]) * c2, bf16_hi(fq[w]) * bf16_hi(fk[w]) * c2);
+                const float4 qa = *reinterpret_cast<const float4 *>(qr + 64 * kk), qb = *reinterpret_cast<const float4 *>(qr + 64 * kk + 16);
+                const u32x4 fk = ld_lds16(k2r + 32 * kk);
+                A[kk][0] = pack_bf16(qa.x * bf16_lo(fk[0]), qa.y * bf16_hi(fk[0]));
+                A[kk][1] = pack_bf16(qa.z * bf16_lo(fk[1]), qa.w * bf16_hi(fk[1]));
+                A[kk][2] = pack_bf16(qb.x * bf16_lo(fk[2]), qb.y * bf16_hi(fk[2]));
+                A[kk][3] = pack_bf16(qb.z * bf16_lo(fk[3]), qb.w * bf16_hi(fk[3]));
             }
             if constexpr (DQ) {
                 const char *dor = lds + C::DOS + c * PITCH + 16 * hf;
@@ -318,24 +325,33 @@ __global__ __launch_bounds__(512) void bwd_q_kernel(KParams p, float *ws, int ha
         // ---- round end: add into the shared fp32 rows, one d-slice per wave and phase
         {
             if (r + 1 < R) issue_rows(r);      // the rows that the next round adds arrive behind the phases below
-            const char *qr = lds + (DQ ? C::QS : C::DOS) + c * PITCH + 16 * hf * 2;   // factor of the scattered rows
+            // factor of the scattered rows: DQ the fp32 q rows (times scale log2(e): the combine kernel multiplies by ln 2), DV the dO rows
+            const char *qr = DQ ? lds + C::QS + c * C::QPITCH + 16 * hf * 4 : lds + C::DOS + c * PITCH + 16 * hf * 2;
             const char *k2r = lds + C::K2S + slot * PITCH + 16 * hf * 2;
             float *srow_p = sc + slot * C::SPITCH + 16 * hf;
             float *drow_p = dqs + c * C::SPITCH + 16 * hf;
             auto add_slice = [&](auto slice_tag) {
                 constexpr int S = decltype(slice_tag)::value;     // slice: dt = S / 2, registers 8*(S%2) .. +7
                 constexpr int dt = S >> 1, r0 = 8 * (S & 1);
-                const u32x4 xq = ld_lds16(qr + dt * 64 + r0 * 2);
+                float4 x0, x1;
+                if constexpr (DQ) {
+                    x0 = *reinterpret_cast<const float4 *>(qr + (32 * dt + r0) * 4);
+                    x1 = *reinterpret_cast<const float4 *>(qr + (32 * dt + r0) * 4 + 16);
+                } else {
+                    const u32x4 xq = ld_lds16(qr + dt * 64 + r0 * 2);
+                    x0 = make_float4(bf16_lo(xq[0]), bf16_hi(xq[0]), bf16_lo(xq[1]), bf16_hi(xq[1]));
+                    x1 = make_float4(bf16_lo(xq[2]), bf16_hi(xq[2]), bf16_lo(xq[3]), bf16_hi(xq[3]));
+                }
                 float *dst = srow_p + 32 * dt + r0;
                 float4 a0 = *reinterpret_cast<float4 *>(dst), a1 = *reinterpret_cast<float4 *>(dst + 4);
-                a0.x += bf16_lo(xq[0]) * acc[dt][r0];
-                a0.y += bf16_hi(xq[0]) * acc[dt][r0 + 1];
-                a0.z += bf16_lo(xq[1]) * acc[dt][r0 + 2];
-                a0.w += bf16_hi(xq[1]) * acc[dt][r0 + 3];
-                a1.x += bf16_lo(xq[2]) * acc[dt][r0 + 4];
-                a1.y += bf16_hi(xq[2]) * acc[dt][r0 + 5];
-                a1.z += bf16_lo(xq[3]) * acc[dt][r0 + 6];
-                a1.w += bf16_hi(xq[3]) * acc[dt][r0 + 7];
+                a0.x += x0.x * acc[dt][r0];
+                a0.y += x0.y * acc[dt][r0 + 1];
+                a0.z += x0.z * acc[dt][r0 + 2];
+                a0.w += x0.w * acc[dt][r0 + 3];
+                a1.x += x1.x * acc[dt][r0 + 4];
+                a1.y += x1.y * acc[dt][r0 + 5];
+                a1.z += x1.z * acc[dt][r0 + 6];
+                a1.w += x1.w * acc[dt][r0 + 7];
                 *reinterpret_cast<float4 *>(dst) = a0;
                 *reinterpret_cast<float4 *>(dst + 4) = a1;
                 if constexpr (DQ) {
@@ -470,7 +486,7 @@ __global__ __launch_bounds__(256) void dk2_dv2_combine_kernel(KParams p, const f
     u32x4 ok, ov;
 #pragma unroll
     for (int w = 0; w < 4; ++w) {
-        ok[w] = pack_bf16(ak[2 * w] * p.scale, ak[2 * w + 1] * p.scale);
+        ok[w] = pack_bf16(ak[2 * w] * kLn2, ak[2 * w + 1] * kLn2);   // the partial rows carry q * scale * log2(e)
         ov[w] = pack_bf16(av[2 * w], av[2 * w + 1]);
     }
     st_global16(p.dk2.ptr + b * p.dk2.sb + (int64_t)k * p.dk2.sn + hk * p.dk2.sh + piece * 16, ok);

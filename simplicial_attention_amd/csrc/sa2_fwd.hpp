@@ -52,9 +52,10 @@ struct FwdCfg {
     static constexpr int APITCH = D + 4;              // floats per row of the shared accumulator
     static constexpr int ACC = 32 * APITCH * 4;
     static constexpr int EXCH = 8 * 32 * 4;           // one float per (wave, row)
-    static constexpr int QS = RING + ACC + 2 * EXCH;  // q rows of the tile      [32][PITCH]
+    static constexpr int QS = RING + ACC + 2 * EXCH;  // q rows of the tile times scale log2(e), fp32 [32][QPITCH bytes]
+    static constexpr int QPITCH = D * 4 + 16;
     static constexpr int KSLOTS = 64;                 // circular k2 / v2 rows
-    static constexpr int K2S = QS + TILE;
+    static constexpr int K2S = QS + 32 * QPITCH;
     static constexpr int V2S = K2S + KSLOTS * PITCH;
     static constexpr int MASKS = V2S + KSLOTS * PITCH; // additive masks (0 / -inf) of the diagonal tile and of up to two lower-edge tiles
     static constexpr int MASK = 16 * 64 * 4;          // one table: [4 quarters][64 lanes][4 floats]
@@ -145,7 +146,13 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
             const int row = x / PPR, col = (x % PPR) * 16;
             int ii = i0 + row;
             ii = ii < N ? ii : N - 1;
-            *reinterpret_cast<u32x4 *>(lds + C::QS + row * PITCH + col) = ld_global16(qg + (int64_t)ii * p.q.sn + col);
+            // unpacked and scaled once per workgroup: the operand build of every offset then multiplies without
+            // unpacking or scaling q again
+            const u32x4 fq = ld_global16(qg + (int64_t)ii * p.q.sn + col);
+            const float c2 = p.scale_log2e;
+            float4 *dst = reinterpret_cast<float4 *>(lds + C::QS + row * C::QPITCH + col * 2);
+            dst[0] = make_float4(bf16_lo(fq[0]) * c2, bf16_hi(fq[0]) * c2, bf16_lo(fq[1]) * c2, bf16_hi(fq[1]) * c2);
+            dst[1] = make_float4(bf16_lo(fq[2]) * c2, bf16_hi(fq[2]) * c2, bf16_lo(fq[3]) * c2, bf16_hi(fq[3]) * c2);
         }
         for (int x = tid; x < 39 * PPR; x += 512) {
             const int row = x / PPR, col = (x % PPR) * 16;
@@ -228,14 +235,15 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
         const int slot = (c - dlt) & 63;              // slot of row k = i - dlt in the circular k2/v2 rows
         {
             const char *k2row = lds + C::K2S + slot * PITCH + 16 * hf;
-            const char *qr = lds + C::QS + c * PITCH + 16 * hf;
-            const float c2 = p.scale_log2e;
+            const char *qr = lds + C::QS + c * C::QPITCH + 32 * hf;
 #pragma unroll
             for (int kk = 0; kk < KS; ++kk) {
-                const u32x4 fq = ld_lds16(qr + 32 * kk), fk = ld_lds16(k2row + 32 * kk);
-#pragma unroll
-                for (int w = 0; w < 4; ++w)
-                    A[kk][w] = pack_bf16(bf16_lo(fq[w]) * bf16_lo(fk[w]) * c2, bf16_hi(fq[w]) * bf16_hi(fk[w]) * c2);
+                const float4 qa = *reinterpret_cast<const float4 *>(qr + 64 * kk), qb = *reinterpret_cast<const float4 *>(qr + 64 * kk + 16);
+                const u32x4 fk = ld_lds16(k2row + 32 * kk);
+                A[kk][0] = pack_bf16(qa.x * bf16_lo(fk[0]), qa.y * bf16_hi(fk[0]));
+                A[kk][1] = pack_bf16(qa.z * bf16_lo(fk[1]), qa.w * bf16_hi(fk[1]));
+                A[kk][2] = pack_bf16(qb.x * bf16_lo(fk[2]), qb.y * bf16_hi(fk[2]));
+                A[kk][3] = pack_bf16(qb.z * bf16_lo(fk[3]), qb.w * bf16_hi(fk[3]));
             }
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) T[dt] = zero16();
@@ -423,8 +431,8 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
                 if (hf == 0) p.m_save[srow_g] = fresh ? 0.f : M;
             }
             Mc = Mn;
-            // the round's contribution of this wave, v2_{i-dlt} * T * g, is formed in place in T before the phases
-            // (nothing there depends on another wave), so that a phase is only: read the slice, add, write, barrier
+            // the round's contribution of this wave is v2_{i-dlt} * T * g: the product with v2 is formed in place in T
+            // before the phases (nothing there depends on another wave), the weight g rides on the phase's multiply-add
             {
                 const char *v2row = lds + C::V2S + slot * PITCH + 16 * hf * 2;
 #pragma unroll
@@ -434,8 +442,8 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
                         const u32x4 xv = ld_lds16(v2row + dt * 64 + half * 16);
 #pragma unroll
                         for (int w = 0; w < 4; ++w) {
-                            T[dt][8 * half + 2 * w] *= bf16_lo(xv[w]) * g;
-                            T[dt][8 * half + 2 * w + 1] *= bf16_hi(xv[w]) * g;
+                            T[dt][8 * half + 2 * w] *= bf16_lo(xv[w]);
+                            T[dt][8 * half + 2 * w + 1] *= bf16_hi(xv[w]);
                         }
                     }
             }
@@ -449,14 +457,14 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
                     a0.x *= fo; a0.y *= fo; a0.z *= fo; a0.w *= fo;
                     a1.x *= fo; a1.y *= fo; a1.z *= fo; a1.w *= fo;
                 }
-                a0.x += T[dt][r0];
-                a0.y += T[dt][r0 + 1];
-                a0.z += T[dt][r0 + 2];
-                a0.w += T[dt][r0 + 3];
-                a1.x += T[dt][r0 + 4];
-                a1.y += T[dt][r0 + 5];
-                a1.z += T[dt][r0 + 6];
-                a1.w += T[dt][r0 + 7];
+                a0.x += T[dt][r0] * g;
+                a0.y += T[dt][r0 + 1] * g;
+                a0.z += T[dt][r0 + 2] * g;
+                a0.w += T[dt][r0 + 3] * g;
+                a1.x += T[dt][r0 + 4] * g;
+                a1.y += T[dt][r0 + 5] * g;
+                a1.z += T[dt][r0 + 6] * g;
+                a1.w += T[dt][r0 + 7] * g;
                 *reinterpret_cast<float4 *>(dst) = a0;
                 *reinterpret_cast<float4 *>(dst + 4) = a1;
             };
