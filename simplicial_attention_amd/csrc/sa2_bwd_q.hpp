@@ -107,7 +107,7 @@ __global__ __launch_bounds__(512) void bwd_q_kernel(KParams p, float *ws, int ha
     // ---- ring staging: direct-to-LDS loads, wave w moves chunk w of the K1 tile and of the V1 tile (D = 64: four
     // chunks per tile, waves 0-3 stage)
     using RT = typename C::RT;
-    const bool stager = wave < RT::NCH;
+    const bool stager = RT::NCH >= 8 || wave < RT::NCH;
     const int st_row = RT::st_row(wave % RT::NCH, lane), st_col = RT::st_col(lane);
     int n_load = 0, u_load = 0;
     // address = tile base (uniform) + this lane's row and column (32 bits); only the diagonal tile can
@@ -116,17 +116,23 @@ __global__ __launch_bounds__(512) void bwd_q_kernel(KParams p, float *ws, int ha
     const uint32_t so_k = (uint32_t)(st_row * (int)p.k1.sn + st_col), so_v = (uint32_t)(st_row * (int)p.v1.sn + st_col);
     const uint32_t so_k_diag = (uint32_t)(st_row_diag * (int)p.k1.sn + st_col), so_v_diag = (uint32_t)(st_row_diag * (int)p.v1.sn + st_col);
     const uint32_t lds_chunk = (uint32_t)(uintptr_t)lds + (wave % RT::NCH) * RT::CP;
+    // tile bases as running pointers (t_lo, t_lo + 1, ..., t_hi, then t_lo again: no multiplications in the step).
+    // Loads are issued at every step, also behind the last tile (the sequence runs on into a buffer that no wave
+    // reads any more), so the step has no branch on its position; the kernel waits for the last ones before it ends.
+    const char *const k_low = k1g + (int64_t)(32 * t_lo) * p.k1.sn, *const v_low = v1g + (int64_t)(32 * t_lo) * p.v1.sn;
+    const int64_t k_step = 32 * p.k1.sn, v_step = 32 * p.v1.sn;
+    const char *kb = k_low, *vb = v_low;
     auto issue_loads = [&]() {
-        const int t = t_lo + n_load;
-        const char *kb = k1g + (int64_t)(32 * t) * p.k1.sn;
-        const char *vb = v1g + (int64_t)(32 * t) * p.v1.sn;
+        const bool diag = n_load == NT - 1;           // the diagonal tile t_hi closes the sequence
         if (stager) {
             const uint32_t dst = lds_chunk + (u_load & 1) * C::BUF;
-            load_to_lds16(kb, t == t_hi ? so_k_diag : so_k, dst);
-            load_to_lds16(vb, t == t_hi ? so_v_diag : so_v, dst + C::OFF_V);
+            load_to_lds16(kb, diag ? so_k_diag : so_k, dst);
+            load_to_lds16(vb, diag ? so_v_diag : so_v, dst + C::OFF_V);
         }
         ++u_load;
-        n_load = (n_load == NT - 1) ? 0 : n_load + 1;
+        kb = diag ? k_low : kb + k_step;
+        vb = diag ? v_low : vb + v_step;
+        n_load = diag ? 0 : n_load + 1;
     };
     const int r_lane = RT::row_lane(lane);            // row fragment: row c, pieces 2*kk + hf
     const int t_lane = RT::tr_lane(lane);             // transposed fragment, per-lane part
@@ -212,7 +218,7 @@ __global__ __launch_bounds__(512) void bwd_q_kernel(KParams p, float *ws, int ha
     auto open_step = [&]() {
         if (stager) wait_loads<0>();
         __syncthreads();
-        if (u + 1 < U) issue_loads();
+        issue_loads();
     };
 
     const f32x16 neg_delta = splat16(-dl);      // DQ: -delta_i in every element (one query row per lane column)
@@ -381,6 +387,7 @@ __global__ __launch_bounds__(512) void bwd_q_kernel(KParams p, float *ws, int ha
             if (r + 1 < R) flush_rows(24 - 8 * r, 8);
         }
     }
+    wait_loads<0>();           // (the transfer issued behind the last tile still writes into the ring)
     // ---- the rows that the last round leaves: k - i0 = -8 (R - 1) - 7 .. 31 - 8 (R - 1)
     flush_rows(-8 * (R - 1) - 7, 39);
 

@@ -106,7 +106,7 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
 
     // ---- ring staging: direct-to-LDS loads, wave w moves chunk(s) w of the K1 tile and of the V1 tile.  Lane p of a
     // chunk load fetches row (p / 4) % RPC, segment p / (4 RPC), piece p % 4 of the segment
-    const bool stager = wave < C::NCH;                           // D = 64: four chunks per tile, waves 0-3 stage
+    const bool stager = C::NCH >= 8 || wave < C::NCH;            // D = 64: four chunks per tile, waves 0-3 stage
     const int st_row = C::RT::st_row(wave % C::NCH, lane), st_col = C::RT::st_col(lane);
     int n_load = 0;                                   // sequence index (within the round) of the next load
     int b_load = 0;                                   // ring buffer of the next load
@@ -116,15 +116,23 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
     const uint32_t so_k = (uint32_t)(st_row * (int)p.k1.sn + st_col), so_v = (uint32_t)(st_row * (int)p.v1.sn + st_col);
     const uint32_t so_k_diag = (uint32_t)(st_row_diag * (int)p.k1.sn + st_col), so_v_diag = (uint32_t)(st_row_diag * (int)p.v1.sn + st_col);
     const uint32_t lds_chunk = (uint32_t)(uintptr_t)lds + (wave % C::NCH) * C::CP;
+    // tile bases as running pointers: the diagonal tile, then t_lo, t_lo + 1, ... (no multiplications in the step)
+    const char *const k_diag = k1g + (int64_t)(32 * t_hi) * p.k1.sn, *const v_diag = v1g + (int64_t)(32 * t_hi) * p.v1.sn;
+    const char *const k_low = k1g + (int64_t)(32 * t_lo) * p.k1.sn, *const v_low = v1g + (int64_t)(32 * t_lo) * p.v1.sn;
+    const int64_t k_step = 32 * p.k1.sn, v_step = 32 * p.v1.sn;
+    const char *kb = k_diag, *vb = v_diag;
+    // Loads are issued at every step, also behind the last tile a round needs (the sequence of tiles simply runs
+    // on, into buffers that no wave reads any more): every step then waits for the same number of transfers and
+    // the step has no branch on the position in the sequence.  The kernel waits for the last ones before it ends.
     auto issue_loads = [&]() {
-        const int t = tile_of(n_load);
-        const char *kb = k1g + (int64_t)(32 * t) * p.k1.sn;
-        const char *vb = v1g + (int64_t)(32 * t) * p.v1.sn;
         if (stager) {
             load_to_lds16(kb, n_load == 0 ? so_k_diag : so_k, lds_chunk + b_load);
             load_to_lds16(vb, n_load == 0 ? so_v_diag : so_v, lds_chunk + b_load + C::DTILE);
         }
-        n_load = (n_load == NT - 1) ? 0 : n_load + 1;
+        const bool wrap = n_load == NT - 1;
+        kb = wrap ? k_diag : (n_load == 0 ? k_low : kb + k_step);
+        vb = wrap ? v_diag : (n_load == 0 ? v_low : vb + v_step);
+        n_load = wrap ? 0 : n_load + 1;
         b_load = (b_load == (C::NBUF - 1) * C::BUF) ? 0 : b_load + C::BUF;
     };
     // K1 fragment kk of row c: segment kk / 2, pieces 2 (kk % 2) + hf
@@ -206,19 +214,16 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
     // u - 1, in which its K1 fragments are read: two steps of time for the memory latency.
     int b_cur = 0, b_nxt = C::BUF;
     issue_loads();
-    if (U > 1) issue_loads();
-    if (U > 2) issue_loads();
+    issue_loads();
+    issue_loads();
     int u = 0;
     wait_loads<0>();
     // start of step u: the tile of step u + 1 has landed (at most the transfers of step u + 2 are still in flight),
     // everything is published, the transfer of step u + 3 starts
     auto open_step = [&]() {
-        if (stager) {
-            if (u + 2 < U) wait_loads<2>();
-            else wait_loads<0>();
-        }
+        if (stager) wait_loads<2>();
         __syncthreads();
-        if (u + 3 < U) issue_loads();
+        issue_loads();
     };
     auto close_step = [&]() {
         b_cur = b_nxt;
@@ -479,6 +484,7 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
         }
     }
 
+    wait_loads<0>();           // (transfers issued behind the last tile still write into the ring)
     // ---- output: O = acc_sh / L with L = sum_w l_w 2^(M_w - Mc)
     {
         auto sw = __builtin_amdgcn_permlane32_swap(as_u32(l), as_u32(l), false, false);
