@@ -220,9 +220,14 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
     wait_loads<0>();
     // start of step u: the tile of step u + 1 has landed (at most the transfers of step u + 2 are still in flight),
     // everything is published, the transfer of step u + 3 starts
-    auto open_step = [&]() {
+    // (work placed right behind a barrier runs with an empty MFMA pipe: the steps issue their loads behind the first
+    // MFMA of the logit chain and prepare the chain's start value ahead of the barrier)
+    auto open_step_barrier = [&]() {
         if (stager) wait_loads<2>();
         __syncthreads();
+    };
+    auto open_step = [&]() {
+        open_step_barrier();
         issue_loads();
     };
     auto close_step = [&]() {
@@ -290,12 +295,15 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
-        auto logit_chain = [&](f32x16 &X) {
+        auto logit_chain = [&](f32x16 &X, auto loads_tag) {
             const char *vbase = lds + b_cur + v_lane;
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int kk = 0; kk < KS; ++kk) {
                 X = mfma32(kf[kk], A[kk], X);
+                if constexpr (decltype(loads_tag)::value) {
+                    if (kk == 0) issue_loads();
+                }
                 const int k2s = kk / DT, dt = kk % DT;
                 vf[dt][k2s][0] = lds_read_tr<D, 0>(vbase + C::RT::tr_imm(16 * k2s, 32 * dt), 0, 0);
                 vf[dt][k2s][1] = lds_read_tr<D, 0>(vbase + C::RT::tr_imm(16 * k2s + 8, 32 * dt), 0, 0);
@@ -338,7 +346,7 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
                 // attends an entry of it, so this is where the rows get their softmax reference M
                 open_step();
                 f32x16 X = zero16();
-                logit_chain(X);
+                logit_chain(X, std::false_type{});
                 {
                     // row j = 32 t + 4 hf + e (e = 8 (rr / 4) + rr % 4) is attended iff 0 <= i - j < w1;
                     // lanes without a valid k2 row get a distance no e can bring into range
@@ -371,7 +379,6 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
             f32x16 NMv = splat16(nm);       // the chains' start value, kept in registers (eight moves per step instead of sixteen)
             u32x4 pb[2];
             for (; n < NT; ++n) {
-                open_step();
                 f32x16 X = NMv;
                 if (n < n_masked) {
                     const char *mk = lds + C::MASKS + n * C::MASK + lane * 16;
@@ -384,7 +391,8 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
                         X[4 * qq + 3] += m4.w;
                     }
                 }
-                logit_chain(X);
+                open_step_barrier();
+                logit_chain(X, std::true_type{});
                 const float l_before = l;
                 exponentials(X, pb);
                 if (__builtin_expect(wave_any(!(l < kBig)), 0)) {
