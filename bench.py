@@ -126,7 +126,7 @@ ENTRY_KERNEL = {'fwd': 'fwd', 'bwd_dq_dk2_pass': 'bwd_q_kernel', 'bwd_dkv1': 'bw
 
 def kernel_symbol(entry, D, w2):
     if entry == 'fwd':
-        return 'sa2::fwd8_kernel<64, 32>' if (D == 64 and w2 <= 32) else 'sa2::fwd_kernel<%d>' % D
+        return 'sa2::fwd_kernel<%d>' % D
     if entry == 'bwd_dq_dk2_pass':
         return 'sa2::bwd_q_kernel<%d, true>' % D
     if entry == 'bwd_dkv1':
@@ -163,7 +163,7 @@ def traffic_from(directory):
         for f in glob.glob(os.path.join(directory, sub, '**', '*counter_collection.csv'), recursive=True):
             for row in csv.DictReader(open(f)):
                 name = row.get('Kernel_Name', '')
-                if kernel_part == 'fwd' and not ('fwd_kernel' in name or 'fwd8_kernel' in name):
+                if kernel_part == 'fwd' and 'fwd_kernel' not in name:
                     continue
                 if row.get('Counter_Name') == counter and kernel_part in name:
                     vals.append(float(row['Counter_Value']))

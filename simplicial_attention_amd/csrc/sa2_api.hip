@@ -17,7 +17,6 @@
 #include "sa2_lds.hpp"
 #include "sa2_qkv_norm.hpp"
 #include "sa2_fwd.hpp"
-#include "sa2_fwd8.hpp"
 
 namespace {
 
@@ -192,10 +191,7 @@ int sa2_fwd(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, 
         k.m_save = saved->m;
     }
     const int grid = prob->batch * prob->heads * ((prob->seq_len + 31) / 32);
-    // dim_head 64 with a second window of up to 32: the instance that fits four waves per SIMD
-    // (two workgroups per CU); everything else: the general kernel (any second window)
-    if (prob->dim_head == 64 && prob->w2 <= 32) hipLaunchKernelGGL((sa2::fwd8_kernel<64, 32>), dim3(grid), dim3(512), 0, s, k);
-    else SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL(sa2::fwd_kernel<DH>, dim3(grid), dim3(512), 0, s, k));
+    SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL(sa2::fwd_kernel<DH>, dim3(grid), dim3(512), 0, s, k));
     return after_launch("forward");
 }
 

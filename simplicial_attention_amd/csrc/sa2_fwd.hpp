@@ -52,21 +52,29 @@ struct FwdCfg {
     static constexpr int APITCH = D + 4;              // floats per row of the shared accumulator
     static constexpr int ACC = 32 * APITCH * 4;
     static constexpr int EXCH = 8 * 32 * 4;           // one float per (wave, row)
-    static constexpr int QS = RING + ACC + 2 * EXCH;  // q rows of the tile times scale log2(e), fp32 [32][QPITCH bytes]
-    static constexpr int QPITCH = D * 4 + 16;
+    // q rows of the tile [32][QPITCH bytes]: fp32 times scale log2(e); at D = 64 bf16 (the instance then fits 80 KiB of
+    // LDS and 128 registers: two workgroups per CU)
+    static constexpr bool QF = D != 64;
+    // waves per SIMD the instance is compiled for: D = 128 needs 236 registers (one workgroup per CU); D = 64 is held
+    // to 128 registers (a few spills outside the step's MFMA blocks) so that two workgroups share a CU, which is worth
+    // 20 % at D = 64; D = 32 fits by itself
+    static constexpr int WPE = D == 128 ? 2 : 4;
+    static constexpr int QS = RING + ACC + 2 * EXCH;
+    static constexpr int QPITCH = QF ? D * 4 + 16 : tile_pitch<D>();
     static constexpr int KSLOTS = 64;                 // circular k2 / v2 rows
     static constexpr int K2S = QS + 32 * QPITCH;
     static constexpr int V2S = K2S + KSLOTS * PITCH;
     static constexpr int MASKS = V2S + KSLOTS * PITCH; // additive masks (0 / -inf) of the diagonal tile and of up to two lower-edge tiles
     static constexpr int MASK = 16 * 64 * 4;          // one table: [4 quarters][64 lanes][4 floats]
     static constexpr int LDS = MASKS + 3 * MASK;
+    static_assert(D == 128 || 2 * LDS <= 160 * 1024, "two workgroups per CU need half the LDS each");
     static_assert(RING - CP < 65536, "the LDS address of a direct load travels in 16 bits of M0");
     static constexpr int PPR = D / 8;                 // 16-byte pieces per row
     static constexpr int PIECES = 32 * PPR;           // ... per tile
 };
 
 template <int D>
-__global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(FwdCfg<D>::WPE, FwdCfg<D>::WPE))) void fwd_kernel(KParams p) {
     using C = FwdCfg<D>;
     constexpr int KS = C::KS, DT = C::DT, PPR = C::PPR, PITCH = C::PITCH;
     constexpr float kBig = 1.2379400392853803e27f;    // 2^90: row sums beyond it move the reference
@@ -154,13 +162,17 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
             const int row = x / PPR, col = (x % PPR) * 16;
             int ii = i0 + row;
             ii = ii < N ? ii : N - 1;
-            // unpacked and scaled once per workgroup: the operand build of every offset then multiplies without
-            // unpacking or scaling q again
             const u32x4 fq = ld_global16(qg + (int64_t)ii * p.q.sn + col);
-            const float c2 = p.scale_log2e;
-            float4 *dst = reinterpret_cast<float4 *>(lds + C::QS + row * C::QPITCH + col * 2);
-            dst[0] = make_float4(bf16_lo(fq[0]) * c2, bf16_hi(fq[0]) * c2, bf16_lo(fq[1]) * c2, bf16_hi(fq[1]) * c2);
-            dst[1] = make_float4(bf16_lo(fq[2]) * c2, bf16_hi(fq[2]) * c2, bf16_lo(fq[3]) * c2, bf16_hi(fq[3]) * c2);
+            if constexpr (C::QF) {
+                // unpacked and scaled once per workgroup: the operand build of every offset then multiplies without
+                // unpacking or scaling q again
+                const float c2 = p.scale_log2e;
+                float4 *dst = reinterpret_cast<float4 *>(lds + C::QS + row * C::QPITCH + col * 2);
+                dst[0] = make_float4(bf16_lo(fq[0]) * c2, bf16_hi(fq[0]) * c2, bf16_lo(fq[1]) * c2, bf16_hi(fq[1]) * c2);
+                dst[1] = make_float4(bf16_lo(fq[2]) * c2, bf16_hi(fq[2]) * c2, bf16_lo(fq[3]) * c2, bf16_hi(fq[3]) * c2);
+            } else {
+                *reinterpret_cast<u32x4 *>(lds + C::QS + row * C::QPITCH + col) = fq;
+            }
         }
         for (int x = tid; x < 39 * PPR; x += 512) {
             const int row = x / PPR, col = (x % PPR) * 16;
@@ -245,15 +257,27 @@ __global__ __launch_bounds__(512) void fwd_kernel(KParams p) {
         const int slot = (c - dlt) & 63;              // slot of row k = i - dlt in the circular k2/v2 rows
         {
             const char *k2row = lds + C::K2S + slot * PITCH + 16 * hf;
-            const char *qr = lds + C::QS + c * C::QPITCH + 32 * hf;
+            if constexpr (C::QF) {
+                const char *qr = lds + C::QS + c * C::QPITCH + 32 * hf;
 #pragma unroll
-            for (int kk = 0; kk < KS; ++kk) {
-                const float4 qa = *reinterpret_cast<const float4 *>(qr + 64 * kk), qb = *reinterpret_cast<const float4 *>(qr + 64 * kk + 16);
-                const u32x4 fk = ld_lds16(k2row + 32 * kk);
-                A[kk][0] = pack_bf16(qa.x * bf16_lo(fk[0]), qa.y * bf16_hi(fk[0]));
-                A[kk][1] = pack_bf16(qa.z * bf16_lo(fk[1]), qa.w * bf16_hi(fk[1]));
-                A[kk][2] = pack_bf16(qb.x * bf16_lo(fk[2]), qb.y * bf16_hi(fk[2]));
-                A[kk][3] = pack_bf16(qb.z * bf16_lo(fk[3]), qb.w * bf16_hi(fk[3]));
+                for (int kk = 0; kk < KS; ++kk) {
+                    const float4 qa = *reinterpret_cast<const float4 *>(qr + 64 * kk), qb = *reinterpret_cast<const float4 *>(qr + 64 * kk + 16);
+                    const u32x4 fk = ld_lds16(k2row + 32 * kk);
+                    A[kk][0] = pack_bf16(qa.x * bf16_lo(fk[0]), qa.y * bf16_hi(fk[0]));
+                    A[kk][1] = pack_bf16(qa.z * bf16_lo(fk[1]), qa.w * bf16_hi(fk[1]));
+                    A[kk][2] = pack_bf16(qb.x * bf16_lo(fk[2]), qb.y * bf16_hi(fk[2]));
+                    A[kk][3] = pack_bf16(qb.z * bf16_lo(fk[3]), qb.w * bf16_hi(fk[3]));
+                }
+            } else {
+                const char *qr = lds + C::QS + c * C::QPITCH + 16 * hf;
+                const float c2 = p.scale_log2e;
+#pragma unroll
+                for (int kk = 0; kk < KS; ++kk) {
+                    const u32x4 fq = ld_lds16(qr + 32 * kk), fk = ld_lds16(k2row + 32 * kk);
+#pragma unroll
+                    for (int w = 0; w < 4; ++w)
+                        A[kk][w] = pack_bf16(bf16_lo(fq[w]) * c2 * bf16_lo(fk[w]), bf16_hi(fq[w]) * c2 * bf16_hi(fk[w]));
+                }
             }
 #pragma unroll
             for (int dt = 0; dt < DT; ++dt) T[dt] = zero16();
