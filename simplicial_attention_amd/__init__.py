@@ -1,6 +1,6 @@
 """MI355X-native sliding-window 2-simplicial attention (gfx950 HIP kernels behind the
 Python API of lucidrains/simplicial-attention for that one path)."""
-from .naive import naive_two_simplicial_attend
+from .naive import naive_two_simplicial_attend, nth_order_attend, signed_determinant
 from .simplicial_mha import HigherOrderAttention, TwoSimplicialMHA
 from .two_simplicial_attention import (
     SlidingTwoSimplicialAttention,
@@ -10,6 +10,8 @@ from .two_simplicial_attention import (
 
 __all__ = [
     'naive_two_simplicial_attend',
+    'nth_order_attend',
+    'signed_determinant',
     'HigherOrderAttention',
     'TwoSimplicialMHA',
     'SlidingTwoSimplicialAttention',

@@ -13,7 +13,7 @@ from typing import Callable
 import torch
 from torch import nn
 
-from .naive import naive_two_simplicial_attend
+from .naive import naive_two_simplicial_attend, nth_order_attend
 
 
 class HigherOrderAttention(nn.Module):
@@ -59,10 +59,11 @@ class HigherOrderAttention(nn.Module):
         self.to_qkv = nn.Linear(dim, sum(self.split_dims), bias=False)
         self.combine_heads = nn.Linear(heads * dim_head_values, dim, bias=False)
 
+        # more than two key/value sets go to the n-th order attend (simplicial_mha.py:94-98 of the reference, which
+        # like this build refuses the causal flag there)
+        assert not (causal and self.kv_sets > 2), 'the n-th order attend is used without a causal mask, as in the reference'
         if attend is None:
-            if self.kv_sets != 2:
-                raise NotImplementedError('only two key/value sets have a built-in attend; pass attend=...')
-            attend = naive_two_simplicial_attend
+            attend = naive_two_simplicial_attend if self.kv_sets <= 2 else nth_order_attend
         if causal:
             attend = partial(attend, causal=causal)
         self.attend = attend

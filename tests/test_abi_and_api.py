@@ -251,3 +251,66 @@ def test_saved_partials_budget_is_global_per_device(monkeypatch):
     monkeypatch.setenv('SA2_SAVE_PARTIALS_MAX_GIB', '16')
     monkeypatch.setenv('SA2_SAVE_PARTIALS_TOTAL_FRACTION', '0.01')
     assert not _PartialsBudget().admit(3 * gib, 'cuda:0', info)
+
+
+def test_signed_determinant_is_the_triple_product_of_channel_triples():
+    """simplicial_attention.py:36-76: every triple of channels contributes det[q; k1; k2]; pinned against
+    torch.linalg.det, with left-over channels contributing their plain trilinear product."""
+    from simplicial_attention_amd.naive import signed_determinant, naive_two_simplicial_attend
+    g = torch.Generator().manual_seed(5)
+    b, h, n, d = 1, 2, 5, 8                      # two triples and two left-over channels
+    q, k1, k2 = (torch.randn(b, h, n, d, generator=g, dtype=torch.float64) for _ in range(3))
+    got = signed_determinant(q, k1, k2)
+    want = torch.zeros(b, h, n, n, n, dtype=torch.float64)
+    for i in range(n):
+        for j in range(n):
+            for k in range(n):
+                for t in range(d // 3):
+                    m = torch.stack([q[:, :, i, 3 * t:3 * t + 3], k1[:, :, j, 3 * t:3 * t + 3], k2[:, :, k, 3 * t:3 * t + 3]], dim=-2)
+                    want[:, :, i, j, k] += torch.linalg.det(m)
+                want[:, :, i, j, k] += (q[:, :, i, 6:] * k1[:, :, j, 6:] * k2[:, :, k, 6:]).sum(-1)
+    assert torch.allclose(got, want, atol=1e-10)
+    # antisymmetric in the two key sets on the full triples
+    q6, a6, b6 = q[..., :6], k1[..., :6], k2[..., :6]
+    assert torch.allclose(signed_determinant(q6, a6, b6), -signed_determinant(q6, b6, a6).transpose(-1, -2), atol=1e-10)
+    v1, v2 = (torch.randn(b, h, n, d, generator=g, dtype=torch.float64) for _ in range(2))
+    out = naive_two_simplicial_attend(q, (k1, k2), (v1, v2), causal=True, use_signed_determinant=True)
+    assert out.shape == (b, h, n, d) and torch.isfinite(out).all()
+
+
+def test_nth_order_attend_special_cases():
+    """simplicial_attention.py:131-198: one key/value set is ordinary attention (pinned against
+    scaled_dot_product_attention), two sets are the 2-simplicial attend, three sets are pinned by loops."""
+    from simplicial_attention_amd.naive import nth_order_attend, naive_two_simplicial_attend
+    g = torch.Generator().manual_seed(6)
+    b, h, hk, n, d = 2, 4, 2, 6, 8
+    q = torch.randn(b, h, n, d, generator=g, dtype=torch.float64)
+    ks = [torch.randn(b, hk, n, d, generator=g, dtype=torch.float64) for _ in range(3)]
+    vs = [torch.randn(b, hk, n, d, generator=g, dtype=torch.float64) for _ in range(3)]
+    for causal in (False, True):
+        one = nth_order_attend(q, ks[:1], vs[:1], causal=causal)
+        sdpa = torch.nn.functional.scaled_dot_product_attention(q, ks[0].repeat_interleave(2, 1), vs[0].repeat_interleave(2, 1), is_causal=causal)
+        assert torch.allclose(one, sdpa, atol=1e-10)
+        two = nth_order_attend(q, ks[:2], vs[:2], causal=causal)
+        assert torch.allclose(two, naive_two_simplicial_attend(q, ks[:2], vs[:2], causal=causal), atol=1e-10)
+    three = nth_order_attend(q, ks, vs)
+    want = torch.zeros_like(three)
+    for bi in range(b):
+        for hi in range(h):
+            kh = hi // 2
+            for i in range(n):
+                logits = torch.einsum('d,jd,kd,ld->jkl', q[bi, hi, i] * d ** -0.5, ks[0][bi, kh], ks[1][bi, kh], ks[2][bi, kh])
+                w = logits.flatten().softmax(0).view_as(logits)
+                want[bi, hi, i] = torch.einsum('jkl,jd,kd,ld->d', w, vs[0][bi, kh], vs[1][bi, kh], vs[2][bi, kh])
+    assert torch.allclose(three, want, atol=1e-10)
+
+
+def test_module_with_three_key_value_sets_uses_the_nth_order_attend():
+    import simplicial_attention_amd as S
+    torch.manual_seed(0)
+    m = S.HigherOrderAttention(dim=32, dim_head=8, heads=2, number_key_value_sets=3)
+    assert m.attend is S.nth_order_attend
+    out = m(torch.randn(1, 5, 32))
+    assert out.shape == (1, 5, 32) and torch.isfinite(out).all()
+    with pytest.raises(AssertionError):
+        S.HigherOrderAttention(dim=32, dim_head=8, heads=2, number_key_value_sets=3, causal=True)
