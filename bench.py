@@ -2,7 +2,7 @@
 """Benchmark of sliding-window 2-simplicial attention on one MI355X.
 
 One step = one forward + backward of the raw kernel path over one batch of synthetic
-input (BASELINE config 3: B=4, H=8, N=8192, D=128, w1=512, w2=32, bf16; q, k1, k2, v1,
+input (benchmark config 3: B=4, H=8, N=8192, D=128, w1=512, w2=32, bf16; q, k1, k2, v1,
 v2 ~ N(0,1)/sqrt(D), dO ~ N(0,1)), called through the autograd Function with inputs
 resident in HBM.  Prints one JSON line.
 
@@ -59,7 +59,7 @@ def cpu_baseline(N, D, w1, w2, slices, runs=3, naive_runs=5):
 
     `value`: the banded oracle, forward + backward, on `slices` complete (batch, head) slices
              of the benchmarked workload; median of `runs` runs.
-    `naive_config1`: the dense naive attend at BASELINE config 1 (B=1, H=4, N=128, D=32, causal,
+    `naive_config1`: the dense naive attend at benchmark config 1 (B=1, H=4, N=128, D=32, causal,
              N(0,1) inputs), forward and forward + backward through autograd; median of
              `naive_runs` runs each.  This is the reference's own CPU-runnable case.
     """
@@ -226,7 +226,7 @@ def main():
     B, H, HK, N, D, w1, w2 = WORKLOADS[args.workload]
     dev = torch.device('cuda:0')
     if args.only == 'train_cfg5':
-        # BASELINE config 5: one training step (forward, loss, backward, Adam) of the byte-level LM: depth 12,
+        # benchmark config 5: one training step (forward, loss, backward, Adam) of the byte-level LM: depth 12,
         # dim 512, 8 heads of 64 (4 key/value heads), every 2nd layer simplicial (w1=512, w2=32), batch 8 x 2048
         from simplicial_attention_amd.two_simplicial_transformer import TwoSimplicialLM
         torch.manual_seed(4)
@@ -271,7 +271,7 @@ def main():
                           'simplicial_cores_share_of_step': round(6 * core_ms / step_ms, 3), 'steps': args.steps}))
         return
     if args.only == 'module_cfg2':
-        # BASELINE config 2: the multi-head module, tokens (2, 1024, 512), dim_head 64, 8 heads, forward,
+        # benchmark config 2: the multi-head module, tokens (2, 1024, 512), dim_head 64, 8 heads, forward,
         # with and without the fused split + RMSNorm kernel; and that kernel alone at the config-3 token count
         from simplicial_attention_amd import SlidingWindowTwoSimplicialMHA
         from simplicial_attention_amd.qkv_norm import FusedQKVNorm

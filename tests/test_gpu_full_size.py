@@ -119,7 +119,7 @@ def test_config4_one_slice_against_oracle():
 
 
 def test_config1_full_causal_against_dense_naive_attend():
-    """BASELINE config 1 on the HIP path: B=1, H=4, N=128, D=32, float32 N(0,1) inputs from a
+    """benchmark config 1 on the HIP path: B=1, H=4, N=128, D=32, float32 N(0,1) inputs from a
     fixed seed, full causal (both windows = N, the case of the reference's test_triton.py:65-80),
     output and the autograd gradients of all five inputs against the dense naive attend
     (simplicial_attention.py:78-127 restated in oracle/reference_attend.py, layout b h n d).

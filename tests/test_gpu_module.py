@@ -26,7 +26,7 @@ def _pair(dim, heads, kv_heads, dim_head, w1, w2, seed, dim_head_values=None):
 
 
 def test_module_forward_config2():
-    """BASELINE config 2: tokens (2, 1024, 512), dim_head 64, 8 heads, w1=512, w2=32, bf16, forward."""
+    """benchmark config 2: tokens (2, 1024, 512), dim_head 64, 8 heads, w1=512, w2=32, bf16, forward."""
     hip, ref = _pair(512, 8, 8, 64, 512, 32, seed=1)
     tokens = torch.randn(2, 1024, 512, generator=torch.Generator().manual_seed(1)).bfloat16()
     with torch.no_grad():

@@ -215,7 +215,7 @@ def test_c_restatement_matches_brute_force():
 
 
 def test_config1_shape_fp32_naive_and_grads():
-    """BASELINE config 1: B=1, H=4, N=128, D=32, fp32, causal; the dense naive
+    """benchmark config 1: B=1, H=4, N=128, D=32, fp32, causal; the dense naive
     restatement against the banded oracle with windows >= N, output and five grads."""
     g = torch.Generator().manual_seed(0)
     q, k1, k2, v1, v2, do = [torch.randn(1, 4, 128, 32, generator=g) for _ in range(6)]
