@@ -261,18 +261,6 @@ __global__ __launch_bounds__(512) void bwd_q_kernel(KParams p, float *ws, int ha
             if (wave_on) {
                 const char *sub = lds + (u & 1) * C::BUF;
                 const int t = t_lo + n;
-                f32x16 X = splat16(nl);
-                if (t == t_hi || n < n_head) {
-                    const char *mk = lds + C::MASKS + (t == t_hi ? 0 : 1 + n) * C::MASK + lane * 16;
-#pragma unroll
-                    for (int qq = 0; qq < 4; ++qq) {
-                        const float4 m4 = *reinterpret_cast<const float4 *>(mk + qq * 1024);
-                        X[4 * qq] += m4.x;
-                        X[4 * qq + 1] += m4.y;
-                        X[4 * qq + 2] += m4.z;
-                        X[4 * qq + 3] += m4.w;
-                    }
-                }
                 // The operand fragments of the step form one stream: the K1 row fragments of the logit chain, (DQ) the
                 // V1 row fragments of the dP chain, then the transposed fragments of the accumulating products.  A
                 // window of W fragments is kept in flight: behind every MFMA the fragment W places further down the
@@ -289,8 +277,22 @@ __global__ __launch_bounds__(512) void bwd_q_kernel(KParams p, float *ws, int ha
                     else if constexpr (s < NROW) return RT::row_frag(vb, s - KS);
                     else return RT::tr_frag(tb, (s - NROW) / DT, (s - NROW) % DT);
                 };
+                // (the step's first fragment reads are requested first: the start values of the chains are then set up
+                // while they are in flight, not in front of them)
                 u32x4 f[W];
                 static_for<0, (W < NFR ? W : NFR)>([&](auto s) { f[s] = fragment(s); });
+                f32x16 X = splat16(nl);
+                if (t == t_hi || n < n_head) {
+                    const char *mk = lds + C::MASKS + (t == t_hi ? 0 : 1 + n) * C::MASK + lane * 16;
+#pragma unroll
+                    for (int qq = 0; qq < 4; ++qq) {
+                        const float4 m4 = *reinterpret_cast<const float4 *>(mk + qq * 1024);
+                        X[4 * qq] += m4.x;
+                        X[4 * qq + 1] += m4.y;
+                        X[4 * qq + 2] += m4.z;
+                        X[4 * qq + 3] += m4.w;
+                    }
+                }
                 f32x16 dP = neg_delta;      // DQ: the chain starts from -delta_i, so dP - delta costs no VALU work
                 __builtin_amdgcn_sched_barrier(0);
                 static_for<0, NROW>([&](auto sc_) {
