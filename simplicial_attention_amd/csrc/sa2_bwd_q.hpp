@@ -252,9 +252,10 @@ __global__ __launch_bounds__(512) void bwd_q_kernel(KParams p, float *ws, int ha
                 for (int kk = 0; kk < KS; ++kk) Bv[kk] = mul_bf16x8(ld_lds16(dor + 32 * kk), ld_lds16(v2r + 32 * kk));
             }
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) acc[dt] = zero16();
+            for (int dt = 0; dt < DT; ++dt) acc[dt] = zero16_pairs();
         }
         const float nl = col_ok ? -lse2 : -INFINITY;  // where the logit chains start
+        const f32x2 nl2 = {nl, nl};
 
         for (int n = 0; n < NT; ++n) {
             open_step();
@@ -281,7 +282,7 @@ __global__ __launch_bounds__(512) void bwd_q_kernel(KParams p, float *ws, int ha
                 // while they are in flight, not in front of them)
                 u32x4 f[W];
                 static_for<0, (W < NFR ? W : NFR)>([&](auto s) { f[s] = fragment(s); });
-                f32x16 X = splat16(nl);
+                f32x16 X = splat16_pairs(nl2);
                 if (t == t_hi || n < n_head) {
                     const char *mk = lds + C::MASKS + (t == t_hi ? 0 : 1 + n) * C::MASK + lane * 16;
 #pragma unroll

@@ -107,6 +107,20 @@ __device__ __forceinline__ f32x16 zero16() {
     return z;
 }
 
+// sixteen zeros, written as eight 64-bit moves (for accumulators that are cleared inside a kernel's loops)
+__device__ __forceinline__ f32x16 zero16_pairs() {
+    typedef float f32x2_t __attribute__((ext_vector_type(2)));
+    f32x16 z;
+#pragma unroll
+    for (int r = 0; r < 16; r += 2) {
+        f32x2_t t = {0.f, 0.f};
+        asm("" : "+v"(t));
+        z[r] = t[0];
+        z[r + 1] = t[1];
+    }
+    return z;
+}
+
 
 
 __device__ __forceinline__ bool wave_any(bool pred) { return __builtin_amdgcn_ballot_w64(pred) != 0ull; }

@@ -280,7 +280,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(FwdCfg<D>::
                 }
             }
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) T[dt] = zero16();
+            for (int dt = 0; dt < DT; ++dt) T[dt] = zero16_pairs();
         }
 
         // exponentials and row sums of the tile whose referenced logits are in X
@@ -369,7 +369,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(FwdCfg<D>::
                 // ---- the wave's very first step, the diagonal tile of its first offset: every valid row
                 // attends an entry of it, so this is where the rows get their softmax reference M
                 open_step();
-                f32x16 X = zero16();
+                f32x16 X = zero16_pairs();
                 logit_chain(X, std::false_type{});
                 {
                     // row j = 32 t + 4 hf + e (e = 8 (rr / 4) + rr % 4) is attended iff 0 <= i - j < w1;

@@ -148,4 +148,19 @@ __device__ __forceinline__ f32x16 splat16(float x) {
     return r;
 }
 
+
+// the same from a register pair that already holds (x, x): eight 64-bit moves instead of sixteen 32-bit ones
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ f32x16 splat16_pairs(f32x2 xx) {
+    f32x16 r;
+#pragma unroll
+    for (int e = 0; e < 16; e += 2) {
+        f32x2 t = xx;
+        asm("" : "+v"(t));
+        r[e] = t[0];
+        r[e + 1] = t[1];
+    }
+    return r;
+}
+
 }  // namespace sa2
