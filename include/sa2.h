@@ -75,7 +75,8 @@ typedef struct sa2_tensor {
 /* Optional by-products of the forward that the backward can reuse instead of
  * recomputing them (the reference keeps only q, k, v, out and lse for its backward,
  * triton_two_simplicial_attention.py:800-805, and recomputes everything else):
- *   t  bf16 [batch][heads][w2][seq_len][dim_head]:  T[b,h,d,i,:] = sum_j 2^(x_ij - m) v1[j,:]
+ *   t  bf16 [batch][heads][w2][ceil(seq_len/32)] blocks of [32 rows][dim_head], the 16-byte pieces of a block in the
+ *      order the forward's lanes hold them (opaque to the caller):  T[b,h,d,i,:] = sum_j 2^(x_ij - m) v1[j,:]
  *      for the offset d = i - k, x = scaled logit * log2(e)
  *   m  fp32 [batch][heads][w2][seq_len]:            the reference m of that sum
  * With them dV2[k] = sum_d dO[k+d] * T[d,k+d] * 2^(m - lse*log2e) needs no contraction

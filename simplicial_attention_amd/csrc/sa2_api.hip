@@ -155,7 +155,7 @@ static int check_saved(const sa2_saved *saved) {
 
 int64_t sa2_saved_t_bytes(const sa2_problem *prob) {
     if (check_problem(prob) != SA2_OK) return -1;
-    return (int64_t)prob->batch * prob->heads * prob->w2 * prob->seq_len * prob->dim_head * 2;
+    return (int64_t)prob->batch * prob->heads * prob->w2 * ((prob->seq_len + 31) / 32) * 32 * prob->dim_head * 2;
 }
 
 int64_t sa2_saved_m_bytes(const sa2_problem *prob) {
@@ -299,9 +299,8 @@ int sa2_bwd_dq_dkv2(const sa2_problem *prob, const sa2_tensor *q, const sa2_tens
     SA2_TRY(after_launch("dq/dk2/dv2"));
     if (pass == 1) return SA2_OK;    // profiling build, one pass: leave the reductions out of its timing
     if (use_saved) {
-        const int rpb = 256 / (prob->dim_head / 8);
-        const int dgrid = prob->batch * prob->kv_heads * ((prob->seq_len + rpb - 1) / rpb);
-        SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL(sa2::dv2_from_saved_kernel<DH>, dim3(dgrid), dim3(256), 0, s, k));
+        const int dgrid = prob->batch * prob->kv_heads * ((prob->seq_len + 31) / 32);
+        SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL(sa2::dv2_from_saved_kernel<DH>, dim3(dgrid), dim3(sa2::Dv2Cfg<DH>::THREADS), 0, s, k));
         SA2_TRY(after_launch("dv2 from saved partials"));
     }
     const int64_t rows = (int64_t)prob->batch * prob->kv_heads * prob->seq_len;

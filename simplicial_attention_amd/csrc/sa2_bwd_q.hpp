@@ -423,42 +423,73 @@ __global__ __launch_bounds__(512) void bwd_q_kernel(KParams p, float *ws, int ha
 
 // dV2 from the forward's saved per-offset T:
 //     dv2[b,k,hk,:] = sum_g sum_dlt do[b,k+dlt,h,:] * T[b,h,dlt,k+dlt,:] * 2^(m[b,h,dlt,k+dlt] - lse2[b,h,k+dlt])
-// (h = hk*G + g).  Streams T once from HBM; a thread owns 8 d of one row k.
+// (h = hk*G + g).  Streams T once from HBM.  A workgroup owns 32 rows k, a thread 8 d of one row; consecutive
+// threads own consecutive rows, whose pieces are consecutive in the blocked layout of T (saved_t_offset).  The do
+// rows k0 .. k0 + 62 that 32 offsets reach and the 32 x 32 weights are staged in LDS per block of 32 offsets.
 template <int D>
-__global__ __launch_bounds__(256) void dv2_from_saved_kernel(KParams p) {
-    constexpr int LP = D / 8;                 // threads per row
-    constexpr int RPB = 256 / LP;             // rows per block
+struct Dv2Cfg {
+    static constexpr int LP = D / 8;                 // 16-byte pieces per row
+    static constexpr int THREADS = 32 * LP;
+    static constexpr int PITCH = tile_pitch<D>();
+};
+
+template <int D>
+__global__ __launch_bounds__(Dv2Cfg<D>::THREADS) void dv2_from_saved_kernel(KParams p) {
+    using C = Dv2Cfg<D>;
+    constexpr int LP = C::LP, NTH = C::THREADS, PITCH = C::PITCH;
+    __shared__ __attribute__((aligned(16))) char dos[63 * PITCH];
+    __shared__ float wsh[32 * 32];
     const int N = p.N;
-    const int nblk = (N + RPB - 1) / RPB;
-    const int blk = blockIdx.x % nblk;
-    const int bh = blockIdx.x / nblk;
+    const int ntile = (N + 31) / 32;
+    const int kt = blockIdx.x % ntile;
+    const int bh = blockIdx.x / ntile;
     const int hk = bh % p.HK, b = bh / p.HK;
-    const int k = blk * RPB + threadIdx.x / LP;
-    const int col = (threadIdx.x % LP) * 16;  // byte offset inside a row
-    if (k >= N) return;
+    const int tid = threadIdx.x;
+    const int c = tid & 31, piece = tid >> 5;         // d = 8 piece .. 8 piece + 7
+    const int k0 = 32 * kt, k = k0 + c;
+    const int t_piece = saved_t_offset(0, (piece >> 1) & 1, piece >> 2, piece & 1);
     float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-    const int nd = p.w2 < N - k ? p.w2 : N - k;
+    const int nd = p.w2 < N - k0 ? p.w2 : N - k0;     // offsets that reach a row of the sequence from row k0
     for (int g = 0; g < p.G; ++g) {
         const int h = hk * p.G + g;
         const int64_t bh_row = ((int64_t)b * p.H + h);
-        const char *dog = p.dout.ptr + b * p.dout.sb + h * p.dout.sh + col;
+        const char *dog = p.dout.ptr + b * p.dout.sb + h * p.dout.sh;
         const float *lse = p.lse + bh_row * N;
+        for (int d0 = 0; d0 < nd; d0 += 32) {
+            __syncthreads();
+            for (int x = tid; x < 63 * LP; x += NTH) {
+                const int row = x / LP, pc = x % LP;
+                int i = k0 + d0 + row;
+                i = i < N ? i : N - 1;
+                *reinterpret_cast<u32x4 *>(dos + row * PITCH + pc * 16) = ld_global16(dog + (int64_t)i * p.dout.sn + pc * 16);
+            }
+            for (int x = tid; x < 32 * 32; x += NTH) {
+                const int dl = x >> 5, dlt = d0 + dl, i = k0 + dlt + (x & 31);
+                float w = 0.f;
+                if (dlt < p.w2 && i < N) w = fast_exp2(p.m_save[(bh_row * p.w2 + dlt) * N + i] - lse[i] * kLog2e);
+                wsh[x] = w;
+            }
+            __syncthreads();
+            const int nl = nd - d0 < 32 ? nd - d0 : 32;
 #pragma unroll 8
-        for (int dlt = 0; dlt < nd; ++dlt) {
-            const int i = k + dlt;
-            const int64_t srow = (bh_row * p.w2 + dlt) * N + i;
-            const u32x4 t = ld_global16(p.t_save + srow * (D * 2) + col);
-            const u32x4 o = ld_global16(dog + (int64_t)i * p.dout.sn);
-            const float w = fast_exp2(p.m_save[srow] - lse[i] * kLog2e);
+            for (int dl = 0; dl < nl; ++dl) {
+                // (rows past the end have weight 0; their T is read from the last row, which every offset has written)
+                const int i = k + d0 + dl < N ? k + d0 + dl : N - 1;
+                const int64_t sbh = bh_row * p.w2 + d0 + dl;
+                const u32x4 t = ld_global16(p.t_save + (sbh * ntile + (i >> 5)) * saved_t_block<D>() + t_piece + (i & 31) * 16);
+                const u32x4 o = ld_lds16(dos + (c + dl) * PITCH + piece * 16);
+                const float w = wsh[dl * 32 + c];
 #pragma unroll
-            for (int x = 0; x < 4; ++x) {
-                acc[2 * x] += bf16_lo(o[x]) * bf16_lo(t[x]) * w;
-                acc[2 * x + 1] += bf16_hi(o[x]) * bf16_hi(t[x]) * w;
+                for (int x = 0; x < 4; ++x) {
+                    acc[2 * x] += bf16_lo(o[x]) * bf16_lo(t[x]) * w;
+                    acc[2 * x + 1] += bf16_hi(o[x]) * bf16_hi(t[x]) * w;
+                }
             }
         }
     }
+    if (k >= N) return;
     u32x4 r = {pack_bf16(acc[0], acc[1]), pack_bf16(acc[2], acc[3]), pack_bf16(acc[4], acc[5]), pack_bf16(acc[6], acc[7])};
-    st_global16(p.dv2.ptr + b * p.dv2.sb + (int64_t)k * p.dv2.sn + hk * p.dv2.sh + col, r);
+    st_global16(p.dv2.ptr + b * p.dv2.sb + (int64_t)k * p.dv2.sn + hk * p.dv2.sh + piece * 16, r);
 }
 
 // dK2 / dV2 from the partial rows of the workspace: sums the tiles that reach a row and the query heads of a group.

@@ -31,13 +31,21 @@ struct DevTensor {
     int64_t sb, sn, sh;
 };
 
+// The forward's per-offset T rows are kept in blocks of 32 query rows (one tile of one offset), laid out as the
+// forward's lanes hold them: saved_t_offset is the place of the 16-byte piece d = 32 dt + 16 hf + 8 half + 0..7 of
+// row c in its block (a wave's store of one (dt, half) covers 1 KiB of consecutive bytes)
+template <int D>
+__host__ __device__ constexpr int saved_t_block() { return 32 * D * 2; }
+__host__ __device__ constexpr int saved_t_offset(int c, int hf, int dt, int half) { return (2 * dt + half) * 1024 + (32 * hf + c) * 16; }
+
 struct KParams {
     DevTensor q, k1, k2, v1, v2, o, dout, dq, dk1, dk2, dv1, dv2;
     DevTensor o_lo;       // optional bf16 residual out_fp32 - bf16(out); ptr == nullptr if absent
     float *lse;
     float *delta;
     // optional by-products of the forward, reused by the backward (nullptr if absent):
-    // t_save bf16 [B][H][w2][N][D]: T = sum_j 2^(x_ij - m) v1_j per offset, m_save fp32 [B][H][w2][N]: m
+    // t_save bf16 [B][H][w2][ceil(N/32)] blocks of 32 rows (saved_t_offset): T = sum_j 2^(x_ij - m) v1_j per offset,
+    // m_save fp32 [B][H][w2][N]: m
     char *t_save;
     float *m_save;
     int B, N, H, HK, G;   // G = H / HK query heads per key/value head

@@ -213,6 +213,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(FwdCfg<D>::
         }
     };
 
+    // accumulator clears: as 64-bit moves where registers are plentiful (at four waves per SIMD the register pairs
+    // they need cost more in spilled registers than the moves save)
+    auto clear16 = [] {
+        if constexpr (C::WPE == 2) return zero16_pairs();
+        else return zero16();
+    };
     f32x16 T[DT];
     u32x4 A[KS];
     u32x4 kf[KS];              // K1 fragments of the step about to run (requested at the end of the step before, or at the round's start)
@@ -280,7 +286,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(FwdCfg<D>::
                 }
             }
 #pragma unroll
-            for (int dt = 0; dt < DT; ++dt) T[dt] = zero16_pairs();
+            for (int dt = 0; dt < DT; ++dt) T[dt] = clear16();
         }
 
         // exponentials and row sums of the tile whose referenced logits are in X
@@ -369,7 +375,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(FwdCfg<D>::
                 // ---- the wave's very first step, the diagonal tile of its first offset: every valid row
                 // attends an entry of it, so this is where the rows get their softmax reference M
                 open_step();
-                f32x16 X = zero16_pairs();
+                f32x16 X = clear16();
                 logit_chain(X, std::false_type{});
                 {
                     // row j = 32 t + 4 hf + e (e = 8 (rr / 4) + rr % 4) is attended iff 0 <= i - j < w1;
@@ -450,23 +456,23 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(FwdCfg<D>::
             for (int w = 0; w < 8; ++w) Mn = fmaxf(Mn, xm[w * 32 + c]);
             const float fo = (Mc == -INFINITY) ? 0.f : fast_exp2(Mc - Mn);   // rescale of the old content
             const float g = (fresh || !wave_on) ? 0.f : fast_exp2(M - Mn);   // weight of this wave's T
-            // by-product for the backward: this offset's T and its reference
-            if (p.t_save && row_ok && dlt < p.w2) {
-                const int64_t srow_g = (((int64_t)b * p.H + h) * p.w2 + dlt) * N + i;
-                char *trow = p.t_save + srow_g * (D * 2) + 16 * hf * 2;
+            // by-product for the backward: this offset's T (packed here, stored slice by slice in the phases below: a
+            // wave's stores issued in one go block it for thousands of cycles in front of a barrier) and its reference
+            const bool save = p.t_save && row_ok && dlt < p.w2;
+            // (T goes to one block of 32 rows per offset and tile, in the order the lanes hold it: a store of the wave
+            // covers 1 KiB of consecutive bytes)
+            const int64_t sbh = ((int64_t)b * p.H + h) * p.w2 + dlt;
+            const int64_t srow_g = sbh * N + i;
+            char *trow = p.t_save + (sbh * ntile + tile) * saved_t_block<D>() + saved_t_offset(c, hf, 0, 0);
+            u32x4 pk[2 * DT];
 #pragma unroll
-                for (int dt = 0; dt < DT; ++dt) {
-                    u32x4 lo4, hi4;
+            for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-                    for (int w = 0; w < 4; ++w) {
-                        lo4[w] = pack_bf16(T[dt][2 * w], T[dt][2 * w + 1]);
-                        hi4[w] = pack_bf16(T[dt][8 + 2 * w], T[dt][8 + 2 * w + 1]);
-                    }
-                    st_global16(trow + dt * 64, lo4);
-                    st_global16(trow + dt * 64 + 16, hi4);
+                for (int w = 0; w < 4; ++w) {
+                    pk[2 * dt][w] = pack_bf16(T[dt][2 * w], T[dt][2 * w + 1]);
+                    pk[2 * dt + 1][w] = pack_bf16(T[dt][8 + 2 * w], T[dt][8 + 2 * w + 1]);
                 }
-                if (hf == 0) p.m_save[srow_g] = fresh ? 0.f : M;
-            }
+            if (save && hf == 0) p.m_save[srow_g] = fresh ? 0.f : M;
             Mc = Mn;
             // the round's contribution of this wave is v2_{i-dlt} * T * g: the product with v2 is formed in place in T
             // before the phases (nothing there depends on another wave), the weight g rides on the phase's multiply-add
@@ -504,6 +510,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(FwdCfg<D>::
                 a1.w += T[dt][r0 + 7] * g;
                 *reinterpret_cast<float4 *>(dst) = a0;
                 *reinterpret_cast<float4 *>(dst + 4) = a1;
+                if (save) st_global16(trow + saved_t_offset(0, 0, dt, S & 1), pk[S]);
             };
             // 2 DT slices of eight registers: the waves form 8 / (2 DT) groups that take turns, group g owns the
             // phases 2 DT g .. 2 DT g + 2 DT - 1 and its wave w the slice (w + ph) mod 2 DT in phase ph

@@ -145,7 +145,7 @@ class SlidingTwoSimplicialAttention(Function):
         t_save = m_save = None
         t_bytes = lib.sa2_saved_t_bytes(prob) + lib.sa2_saved_m_bytes(prob)
         if needs_grad and partials_budget.admit(t_bytes, q.device):
-            t_save = torch.empty((batch, heads, w2, seq_len, dim), dtype=q.dtype, device=q.device)
+            t_save = torch.empty(lib.sa2_saved_t_bytes(prob), dtype=torch.uint8, device=q.device)
             m_save = torch.empty((batch, heads, w2, seq_len), dtype=torch.float32, device=q.device)
             partials_budget.track(t_save, t_bytes)
         with torch.cuda.device_of(q):
