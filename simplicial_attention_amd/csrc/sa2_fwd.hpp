@@ -406,10 +406,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(FwdCfg<D>::
             // subtraction code follows it.  A row's reference moves only if its row sum says that weights
             // outgrew the safe range.
             float nm = col_ok ? -M : -INFINITY;
-            f32x16 NMv = splat16(nm);       // the chains' start value, kept in registers (eight moves per step instead of sixteen)
+            // the chains' start value, kept in registers where they are plentiful (eight moves per step instead of sixteen)
+            f32x16 NMv;
+            if constexpr (C::WPE == 2) NMv = splat16(nm);
             u32x4 pb[2];
             for (; n < NT; ++n) {
-                f32x16 X = NMv;
+                f32x16 X;
+                if constexpr (C::WPE == 2) X = NMv;
+                else X = splat16(nm);
                 if (n < n_masked) {
                     const char *mk = lds + C::MASKS + n * C::MASK + lane * 16;
 #pragma unroll
@@ -438,7 +442,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(FwdCfg<D>::
                     const float shift = over ? fmaxf(fmaxf(tmax, e_old), 0.f) : 0.f;
                     shift_reference(shift, fast_exp2(-shift), X);
                     nm = col_ok ? -M : -INFINITY;
-                    NMv = splat16(nm);
+                    if constexpr (C::WPE == 2) NMv = splat16(nm);
                     exponentials(X, pb);
                 }
                 value_products(pb);
