@@ -89,6 +89,10 @@ def test_argument_validation_happens_before_any_launch(lib):
     # saved forward partials: sizes, and NULL members are refused
     assert lib.sa2_saved_t_bytes(good) == 1 * 2 * 32 * 64 * 128 * 2
     assert lib.sa2_saved_m_bytes(good) == 1 * 2 * 32 * 64 * 4
+    # the partials are kept in whole blocks of 32 rows: a ragged sequence length rounds up
+    ragged = _native.problem(1, 65, 2, 2, 128, 16, 32, True, 0.1)
+    assert lib.sa2_saved_t_bytes(ragged) == 1 * 2 * 32 * 96 * 128 * 2
+    assert lib.sa2_saved_m_bytes(ragged) == 1 * 2 * 32 * 65 * 4
     assert lib.sa2_saved_t_bytes(None) == -1
     assert lib.sa2_fwd(good, t, t, t, t, t, t, None, lse, ctypes.byref(_native.Saved(None, None)), None) == 1
     assert lib.sa2_fwd(good, t, t, t, t, t, t, None, lse, ctypes.byref(_native.Saved(0x1004, 0x2000)), None) == 4
