@@ -468,53 +468,38 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(FwdCfg<D>::
             const int64_t sbh = ((int64_t)b * p.H + h) * p.w2 + dlt;
             const int64_t srow_g = sbh * N + i;
             char *trow = p.t_save + (sbh * ntile + tile) * saved_t_block<D>() + saved_t_offset(c, hf, 0, 0);
-            u32x4 pk[2 * DT];
-#pragma unroll
-            for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                for (int w = 0; w < 4; ++w) {
-                    pk[2 * dt][w] = pack_bf16(T[dt][2 * w], T[dt][2 * w + 1]);
-                    pk[2 * dt + 1][w] = pack_bf16(T[dt][8 + 2 * w], T[dt][8 + 2 * w + 1]);
-                }
             if (save && hf == 0) p.m_save[srow_g] = fresh ? 0.f : M;
             Mc = Mn;
-            // the round's contribution of this wave is v2_{i-dlt} * T * g: the product with v2 is formed in place in T
-            // before the phases (nothing there depends on another wave), the weight g rides on the phase's multiply-add
-            {
-                const char *v2row = lds + C::V2S + slot * PITCH + 16 * hf * 2;
-#pragma unroll
-                for (int dt = 0; dt < DT; ++dt)
-#pragma unroll
-                    for (int half = 0; half < 2; ++half) {
-                        const u32x4 xv = ld_lds16(v2row + dt * 64 + half * 16);
-#pragma unroll
-                        for (int w = 0; w < 4; ++w) {
-                            T[dt][8 * half + 2 * w] *= bf16_lo(xv[w]);
-                            T[dt][8 * half + 2 * w + 1] *= bf16_hi(xv[w]);
-                        }
-                    }
-            }
+            // the round's contribution of this wave is v2_{i-dlt} * T * g, formed slice by slice inside the phases (the
+            // products then ride on the latency of the phase's LDS reads)
+            const char *v2row = lds + C::V2S + slot * PITCH + 16 * hf * 2;
             float *arow = acc_sh + c * C::APITCH + 16 * hf;
             auto add_slice = [&](auto slice_tag, bool first) {
                 constexpr int S = decltype(slice_tag)::value;     // slice: dt = S / 2, registers 8*(S%2) .. +7
                 constexpr int dt = S >> 1, r0 = 8 * (S & 1);
                 float *dst = arow + 32 * dt + r0;
                 float4 a0 = *reinterpret_cast<float4 *>(dst), a1 = *reinterpret_cast<float4 *>(dst + 4);
+                const u32x4 xv = ld_lds16(v2row + dt * 64 + (S & 1) * 16);
+                if (save) {
+                    u32x4 pk;
+#pragma unroll
+                    for (int w = 0; w < 4; ++w) pk[w] = pack_bf16(T[dt][r0 + 2 * w], T[dt][r0 + 2 * w + 1]);
+                    st_global16(trow + saved_t_offset(0, 0, dt, S & 1), pk);
+                }
                 if (first) {
                     a0.x *= fo; a0.y *= fo; a0.z *= fo; a0.w *= fo;
                     a1.x *= fo; a1.y *= fo; a1.z *= fo; a1.w *= fo;
                 }
-                a0.x += T[dt][r0] * g;
-                a0.y += T[dt][r0 + 1] * g;
-                a0.z += T[dt][r0 + 2] * g;
-                a0.w += T[dt][r0 + 3] * g;
-                a1.x += T[dt][r0 + 4] * g;
-                a1.y += T[dt][r0 + 5] * g;
-                a1.z += T[dt][r0 + 6] * g;
-                a1.w += T[dt][r0 + 7] * g;
+                a0.x += T[dt][r0] * bf16_lo(xv[0]) * g;
+                a0.y += T[dt][r0 + 1] * bf16_hi(xv[0]) * g;
+                a0.z += T[dt][r0 + 2] * bf16_lo(xv[1]) * g;
+                a0.w += T[dt][r0 + 3] * bf16_hi(xv[1]) * g;
+                a1.x += T[dt][r0 + 4] * bf16_lo(xv[2]) * g;
+                a1.y += T[dt][r0 + 5] * bf16_hi(xv[2]) * g;
+                a1.z += T[dt][r0 + 6] * bf16_lo(xv[3]) * g;
+                a1.w += T[dt][r0 + 7] * bf16_hi(xv[3]) * g;
                 *reinterpret_cast<float4 *>(dst) = a0;
                 *reinterpret_cast<float4 *>(dst + 4) = a1;
-                if (save) st_global16(trow + saved_t_offset(0, 0, dt, S & 1), pk[S]);
             };
             // 2 DT slices of eight registers: the waves form 8 / (2 DT) groups that take turns, group g owns the
             // phases 2 DT g .. 2 DT g + 2 DT - 1 and its wave w the slice (w + ph) mod 2 DT in phase ph
