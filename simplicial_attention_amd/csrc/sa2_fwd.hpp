@@ -460,7 +460,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(FwdCfg<D>::
             for (int w = 0; w < 8; ++w) Mn = fmaxf(Mn, xm[w * 32 + c]);
             const float fo = (Mc == -INFINITY) ? 0.f : fast_exp2(Mc - Mn);   // rescale of the old content
             const float g = (fresh || !wave_on) ? 0.f : fast_exp2(M - Mn);   // weight of this wave's T
-            // by-product for the backward: this offset's T (packed here, stored slice by slice in the phases below: a
+            // by-product for the backward: this offset's T (packed and stored slice by slice in the phases below: a
             // wave's stores issued in one go block it for thousands of cycles in front of a barrier) and its reference
             const bool save = p.t_save && row_ok && dlt < p.w2;
             // (T goes to one block of 32 rows per offset and tile, in the order the lanes hold it: a store of the wave
