@@ -120,13 +120,15 @@ int sa2_fwd(const sa2_problem *prob,
 int sa2_bwd_delta(const sa2_problem *prob, const sa2_tensor *out, const sa2_tensor *out_residual,
                   const sa2_tensor *dout, float *delta, void *hip_stream);
 
-/* Bytes of device workspace the backward needs for this problem (fp32 partial rows of
- * dK2/dV2, one block per 32-row query tile); -1 if the problem is invalid.  The
- * reference has no counterpart: its five fp32 gradient buffers of
- * triton_two_simplicial_attention.py:853-857 play the same role.  The first half holds the
- * dK2 rows, the second half the dV2 rows: a backward call that is given the forward's saved
- * partials (sa2_saved) touches only the first half and accepts half this size. */
+/* Bytes of device workspace the backward needs for this problem; -1 if the problem is invalid.
+ * The reference has no counterpart: its five fp32 gradient buffers of
+ * triton_two_simplicial_attention.py:853-857 play the same role.  The workspace holds the fp32
+ * partial rows of dK2 and dV2 (one block per 32-row query tile; dK2 rows first, the dV2 rows
+ * behind them are not needed when the call is given the forward's saved partials, sa2_saved) and,
+ * once those are spent, for small grids the two fp32 partial results of dK1/dV1 per key slab.
+ * sa2_bwd_workspace_bytes_with_saved() is the size that suffices when saved partials are given. */
 int64_t sa2_bwd_workspace_bytes(const sa2_problem *prob);
+int64_t sa2_bwd_workspace_bytes_with_saved(const sa2_problem *prob);
 
 /* dQ, dK2, dV2.  Replaces both passes of two_simplicial_attn_bwd_kv2q_kernel
  * (triton_two_simplicial_attention.py:938-1004; kernel :515-712; dq :697-699,709;

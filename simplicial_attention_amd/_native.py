@@ -26,7 +26,7 @@ STATUS_NAMES = {
 }
 
 EXPORTS = ('sa2_version', 'sa2_last_error', 'sa2_supported', 'sa2_saved_t_bytes', 'sa2_saved_m_bytes', 'sa2_fwd',
-           'sa2_bwd_delta', 'sa2_bwd_workspace_bytes', 'sa2_bwd_dq_dkv2', 'sa2_bwd_dkv1', 'sa2_bwd',
+           'sa2_bwd_delta', 'sa2_bwd_workspace_bytes', 'sa2_bwd_workspace_bytes_with_saved', 'sa2_bwd_dq_dkv2', 'sa2_bwd_dkv1', 'sa2_bwd',
            'sa2_bwd_noalloc_scratch_bytes', 'sa2_bwd_noalloc',
            'sa2_qkv_norm_fwd', 'sa2_qkv_norm_bwd_workspace_bytes', 'sa2_qkv_norm_bwd')
 
@@ -70,7 +70,7 @@ def _declare(lib: ctypes.CDLL) -> ctypes.CDLL:
     P, T, F, V = ctypes.POINTER(Problem), ctypes.POINTER(TensorArg), ctypes.c_void_p, ctypes.c_void_p
     S = ctypes.POINTER(Saved)
     I64 = ctypes.c_int64
-    for name in ('sa2_saved_t_bytes', 'sa2_saved_m_bytes', 'sa2_bwd_workspace_bytes', 'sa2_qkv_norm_bwd_workspace_bytes',
+    for name in ('sa2_saved_t_bytes', 'sa2_saved_m_bytes', 'sa2_bwd_workspace_bytes', 'sa2_bwd_workspace_bytes_with_saved', 'sa2_qkv_norm_bwd_workspace_bytes',
                  'sa2_bwd_noalloc_scratch_bytes'):
         getattr(lib, name).restype = I64
         getattr(lib, name).argtypes = [P]

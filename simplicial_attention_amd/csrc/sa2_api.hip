@@ -254,9 +254,34 @@ static int bwd_pass_filter() {
 // rows below a 32-row query tile that its offsets reach (offsets run in rounds of eight)
 static int q_halo(int w2) { return 8 * ((w2 + 7) / 8) - 1; }
 
+// partial rows of dK2 and dV2 (the dV2 half is not needed with saved forward partials)
+static int64_t partial_rows_bytes(const sa2_problem *prob) {
+    return sa2::qk2_ws_floats(prob->batch, prob->heads, prob->seq_len, prob->dim_head, 32 + q_halo(prob->w2)) * 4;
+}
+
+// dK1/dV1 with the key slabs' work split over two workgroups each (fp32 partial results, summed by a second kernel):
+// for grids that put fewer than four workgroups on a CU, where whole workgroups of unequal length leave many CUs
+// idle at the end.  Depends on the problem only, so that every entry point with a workspace runs the same kernels.
+static bool dkv1_in_parts(const sa2_problem *prob) {
+    const int64_t grid = (int64_t)prob->batch * prob->kv_heads * ((prob->seq_len + 127) / 128);
+    return grid < 4 * 256;
+}
+
+static int64_t dkv1_parts_bytes(const sa2_problem *prob) {
+    if (!dkv1_in_parts(prob)) return 0;
+    return 2ll * 2 * prob->batch * prob->kv_heads * prob->seq_len * prob->dim_head * 4;
+}
+
+static int64_t max64(int64_t a, int64_t b) { return a > b ? a : b; }
+
 int64_t sa2_bwd_workspace_bytes(const sa2_problem *prob) {
     if (check_problem(prob) != SA2_OK) return -1;
-    return sa2::qk2_ws_floats(prob->batch, prob->heads, prob->seq_len, prob->dim_head, 32 + q_halo(prob->w2)) * 4;
+    return max64(partial_rows_bytes(prob), dkv1_parts_bytes(prob));
+}
+
+int64_t sa2_bwd_workspace_bytes_with_saved(const sa2_problem *prob) {
+    if (check_problem(prob) != SA2_OK) return -1;
+    return max64(partial_rows_bytes(prob) / 2, dkv1_parts_bytes(prob));
 }
 
 int sa2_bwd_dq_dkv2(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
@@ -273,10 +298,10 @@ int sa2_bwd_dq_dkv2(const sa2_problem *prob, const sa2_tensor *q, const sa2_tens
     // the dK2 partial rows are the first half of the workspace, the dV2 partial rows the second: with saved
     // forward partials dV2 needs none
     const bool saved_given = saved != nullptr;
-    const int64_t need = sa2_bwd_workspace_bytes(prob) / (saved_given ? 2 : 1);
+    const int64_t need = partial_rows_bytes(prob) / (saved_given ? 2 : 1);
     if (workspace_bytes < need)
-        return fail(SA2_ERR_BAD_SHAPE, "workspace of %lld bytes is smaller than the %lld bytes this call needs (sa2_bwd_workspace_bytes()%s)",
-                    (long long)workspace_bytes, (long long)need, saved_given ? " / 2 with saved partials" : "");
+        return fail(SA2_ERR_BAD_SHAPE, "workspace of %lld bytes is smaller than the %lld bytes this call needs (sa2_bwd_workspace_bytes%s())",
+                    (long long)workspace_bytes, (long long)need, saved_given ? "_with_saved" : "");
     k.dq = dev(dq);
     k.dk2 = dev(dk2);
     k.dv2 = dev(dv2);
@@ -311,18 +336,33 @@ int sa2_bwd_dq_dkv2(const sa2_problem *prob, const sa2_tensor *q, const sa2_tens
     return after_launch("dk2/dv2 combine");
 }
 
-int sa2_bwd_dkv1(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
-                 const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *dout, const float *lse,
-                 const float *delta, const sa2_tensor *dk1, const sa2_tensor *dv1, void *hip_stream) {
+static int launch_dkv1(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
+                       const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *dout, const float *lse,
+                       const float *delta, const sa2_tensor *dk1, const sa2_tensor *dv1, float *parts, void *hip_stream) {
     sa2::KParams k;
     SA2_TRY(bwd_common(prob, q, k1, k2, v1, v2, dout, lse, delta, &k));
     SA2_TRY(check_tensor(dk1, "dk1"));
     SA2_TRY(check_tensor(dv1, "dv1"));
     k.dk1 = dev(dk1);
     k.dv1 = dev(dv1);
+    k.kv_parts = parts;
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
-    int grid = prob->batch * prob->kv_heads * ((prob->seq_len + 127) / 128);
+    const int grid = prob->batch * prob->kv_heads * ((prob->seq_len + 127) / 128);
     // dim_head 128: the two waves of a slab split the contractions; dim_head 64 and 32: each wave forms both outputs
+    if (parts) {
+        if (prob->dim_head == 128)
+            hipLaunchKernelGGL((sa2::bwd_kv8_kernel<128, sa2::kKvSplit, true>), dim3(2 * grid), dim3(512), 0, s, k);
+        else if (prob->dim_head == 64)
+            hipLaunchKernelGGL((sa2::bwd_kv8_kernel<64, sa2::kKvBoth, true>), dim3(2 * grid), dim3(512), 0, s, k);
+        else
+            hipLaunchKernelGGL((sa2::bwd_kv8_kernel<32, sa2::kKvBoth, true>), dim3(2 * grid), dim3(512), 0, s, k);
+        SA2_TRY(after_launch("dk1/dv1 in parts"));
+        const int64_t rows = (int64_t)prob->batch * prob->kv_heads * prob->seq_len;
+        const int rows_per_block = 256 / (prob->dim_head / 8);
+        const int cgrid = (int)((rows + rows_per_block - 1) / rows_per_block);
+        SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL(sa2::dkv1_parts_combine_kernel<DH>, dim3(cgrid), dim3(256), 0, s, k));
+        return after_launch("dk1/dv1 parts combine");
+    }
     if (prob->dim_head == 128)
         hipLaunchKernelGGL((sa2::bwd_kv8_kernel<128, sa2::kKvSplit>), dim3(grid), dim3(512), 0, s, k);
     else if (prob->dim_head == 64)
@@ -330,6 +370,12 @@ int sa2_bwd_dkv1(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor 
     else
         hipLaunchKernelGGL((sa2::bwd_kv8_kernel<32, sa2::kKvBoth>), dim3(grid), dim3(512), 0, s, k);
     return after_launch("dk1/dv1");
+}
+
+int sa2_bwd_dkv1(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
+                 const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *dout, const float *lse,
+                 const float *delta, const sa2_tensor *dk1, const sa2_tensor *dv1, void *hip_stream) {
+    return launch_dkv1(prob, q, k1, k2, v1, v2, dout, lse, delta, dk1, dv1, nullptr, hip_stream);
 }
 
 int sa2_bwd(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
@@ -340,8 +386,15 @@ int sa2_bwd(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, 
     SA2_TRY(sa2_bwd_delta(prob, out, out_residual, dout, delta_ws, hip_stream));
     SA2_TRY(sa2_bwd_dq_dkv2(prob, q, k1, k2, v1, v2, dout, lse, delta_ws, saved, dq, dk2, dv2, workspace,
                             workspace_bytes, hip_stream));
-    SA2_TRY(sa2_bwd_dkv1(prob, q, k1, k2, v1, v2, dout, lse, delta_ws, dk1, dv1, hip_stream));
-    return SA2_OK;
+    // the partial rows of dK2/dV2 are spent by now: the partial results of split key slabs reuse the workspace
+    float *parts = nullptr;
+    if (dkv1_in_parts(prob)) {
+        if (workspace_bytes < dkv1_parts_bytes(prob))
+            return fail(SA2_ERR_BAD_SHAPE, "workspace of %lld bytes is smaller than the %lld bytes this problem's dk1/dv1 pass needs (sa2_bwd_workspace_bytes())",
+                        (long long)workspace_bytes, (long long)dkv1_parts_bytes(prob));
+        parts = static_cast<float *>(workspace);
+    }
+    return launch_dkv1(prob, q, k1, k2, v1, v2, dout, lse, delta_ws, dk1, dv1, parts, hip_stream);
 }
 
 static int64_t align256(int64_t x) { return (x + 255) & ~int64_t(255); }

@@ -84,7 +84,9 @@ struct Kv8Cfg {
     static_assert((MODE == kKvBoth ? 2 : 1) * RED <= LDS, "final reduction must fit (everything else is dead by then)");
 };
 
-template <int D, int MODE>
+// PARTS: two workgroups per key slab, each walks half of the slab's query tiles and leaves fp32 partial rows in
+// p.kv_parts (for grids that would otherwise put one or two long workgroups on every CU and end on a ragged tail)
+template <int D, int MODE, bool PARTS = false>
 __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     constexpr int KS = D / 16, DT = D / 32, PPR = D / 8;
     using L = Kv8Cfg<D, MODE>;
@@ -95,7 +97,9 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
 
     const int N = p.N;
     const int ntile = (N + 127) / 128;
-    const int item = xcd_contiguous(blockIdx.x, gridDim.x);
+    const int item_all = xcd_contiguous(blockIdx.x, gridDim.x);
+    const int part = PARTS ? item_all & 1 : 0;
+    const int item = PARTS ? item_all >> 1 : item_all;
     const int tile = item % ntile;
     const int bh = item / ntile;
     const int hk = bh % p.HK, b = bh / p.HK;
@@ -132,9 +136,29 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
 #pragma unroll
     for (int dt = 0; dt < (TWO ? DT : 1); ++dt) acc2[dt] = zero16();
 
-    const int it_begin = j0 / 32;
     const int last_i = (j0 + 127 + p.w1 - 1 < N - 1) ? j0 + 127 + p.w1 - 1 : N - 1;
-    const int it_end = last_i / 32;
+    const int it_first = j0 / 32, it_last = last_i / 32;          // the query tiles that reach the slab
+    const int it_half = (it_last - it_first + 2) / 2;             // PARTS: the first part takes the larger half
+    const int it_begin = PARTS && part ? it_first + it_half : it_first;
+    const int it_end = PARTS && !part ? it_first + it_half - 1 : it_last;
+    // where a lane's row of a partial result goes (PARTS)
+    auto part_row = [&](int which) {
+        const int64_t rows = (int64_t)p.B * p.HK * N;
+        return p.kv_parts + ((int64_t)(2 * part + which) * rows + ((int64_t)b * p.HK + hk) * N + j) * D + 16 * hf;
+    };
+    if constexpr (PARTS) {
+        if (it_begin > it_end) {
+            // (a slab with a single query tile: nothing for the second part but its zeros)
+            f32x16 z[DT];
+#pragma unroll
+            for (int dt = 0; dt < DT; ++dt) z[dt] = zero16();
+            if (j_ok && wave < 4) {
+                store_row_f32<DT>(part_row(0), z, 0.f);
+                store_row_f32<DT>(part_row(1), z, 0.f);
+            }
+            return;
+        }
+    }
     const bool wave_active = jw < N;
     const int wit_lo = jw / 32;
     const int wit_hi = ((jw + 31 + p.w1 - 1 < N - 1) ? jw + 31 + p.w1 - 1 : N - 1) / 32;
@@ -502,7 +526,11 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                 build_tables(nb, nbuf);
                 next_pair(nb);
             }
-            if (j_ok) store_row<DT>(p.dv1.ptr + b * p.dv1.sb + (int64_t)j * p.dv1.sn + hk * p.dv1.sh + 16 * hf * 2, acc, 1.f);
+            if constexpr (PARTS) {
+                if (j_ok) store_row_f32<DT>(part_row(1), acc, 1.f);
+            } else {
+                if (j_ok) store_row<DT>(p.dv1.ptr + b * p.dv1.sb + (int64_t)j * p.dv1.sn + hk * p.dv1.sh + 16 * hf * 2, acc, 1.f);
+            }
         } else {
             // ---- S waves: dP - delta for both offsets with a build quarter beside the first chain; after the barrier
             // dS = P (dP - delta) and dK1^T += A^T dS, the second offset's dS formed beside the first offset's products
@@ -554,7 +582,11 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                                 [&](auto x, const u32x4 &fr) { acc[x % DT] = mfma32(fr, pb1[x / DT], acc[x % DT]); });
                 }
             }
-            if (j_ok) store_row<DT>(p.dk1.ptr + b * p.dk1.sb + (int64_t)j * p.dk1.sn + hk * p.dk1.sh + 16 * hf * 2, acc, kLn2);   // A carried scale log2(e)
+            if constexpr (PARTS) {
+                if (j_ok) store_row_f32<DT>(part_row(0), acc, kLn2);
+            } else {
+                if (j_ok) store_row<DT>(p.dk1.ptr + b * p.dk1.sb + (int64_t)j * p.dk1.sn + hk * p.dk1.sh + 16 * hf * 2, acc, kLn2);   // A carried scale log2(e)
+            }
         }
         return;
     }
@@ -673,11 +705,42 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     collect(acc, red);
     char *dk1row = p.dk1.ptr + b * p.dk1.sb + (int64_t)j * p.dk1.sn + hk * p.dk1.sh + 16 * hf * 2;
     char *dv1row = p.dv1.ptr + b * p.dv1.sb + (int64_t)j * p.dv1.sn + hk * p.dv1.sh + 16 * hf * 2;
-    if constexpr (DK) store_row<DT>(dk1row, acc, kLn2);   // A carried scale log2(e)
-    if constexpr (MODE == kKvDv) store_row<DT>(dv1row, acc, 1.f);
-    if constexpr (TWO) {
+    static_assert(!PARTS || TWO || SPLIT, "partial results exist for the kernels that form both outputs");
+    if constexpr (PARTS && TWO) {
+        store_row_f32<DT>(part_row(0), acc, kLn2);
         collect(acc2, red + L::RED / 4);
-        store_row<DT>(dv1row, acc2, 1.f);
+        store_row_f32<DT>(part_row(1), acc2, 1.f);
+    } else if constexpr (!PARTS) {
+        if constexpr (DK) store_row<DT>(dk1row, acc, kLn2);   // A carried scale log2(e)
+        if constexpr (MODE == kKvDv) store_row<DT>(dv1row, acc, 1.f);
+        if constexpr (TWO) {
+            collect(acc2, red + L::RED / 4);
+            store_row<DT>(dv1row, acc2, 1.f);
+        }
+    }
+}
+
+// dK1 and dV1 from the two partial results of the split slabs: a thread sums 8 d of one row
+template <int D>
+__global__ __launch_bounds__(256) void dkv1_parts_combine_kernel(KParams p) {
+    constexpr int LP = D / 8;
+    const int64_t rows = (int64_t)p.B * p.HK * p.N;
+    const int64_t row = (int64_t)blockIdx.x * (256 / LP) + threadIdx.x / LP;
+    if (row >= rows) return;
+    const int piece = threadIdx.x % LP;
+    const int j = (int)(row % p.N);
+    const int hk = (int)((row / p.N) % p.HK);
+    const int b = (int)(row / ((int64_t)p.N * p.HK));
+#pragma unroll
+    for (int which = 0; which < 2; ++which) {
+        const float *a = p.kv_parts + ((int64_t)which * rows + row) * D + piece * 8;
+        const float *c = a + 2 * rows * D;
+        const float4 a0 = *reinterpret_cast<const float4 *>(a), a1 = *reinterpret_cast<const float4 *>(a + 4);
+        const float4 c0 = *reinterpret_cast<const float4 *>(c), c1 = *reinterpret_cast<const float4 *>(c + 4);
+        const u32x4 o = {pack_bf16(a0.x + c0.x, a0.y + c0.y), pack_bf16(a0.z + c0.z, a0.w + c0.w),
+                         pack_bf16(a1.x + c1.x, a1.y + c1.y), pack_bf16(a1.z + c1.z, a1.w + c1.w)};
+        const DevTensor &t = which ? p.dv1 : p.dk1;
+        st_global16(t.ptr + b * t.sb + (int64_t)j * t.sn + hk * t.sh + piece * 16, o);
     }
 }
 

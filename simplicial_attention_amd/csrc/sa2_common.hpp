@@ -52,6 +52,9 @@ struct KParams {
     int w1, w2;
     float scale;          // softmax scale
     float scale_log2e;    // scale * log2(e)
+    // dK1/dV1 computed in two parts per key slab (each part walks half of the slab's query tiles): fp32 partial rows
+    // [part][dk1, dv1][B][HK][N][D], summed by dkv1_parts_combine_kernel; nullptr when the slabs are not split
+    float *kv_parts;
 };
 
 // compile-time loop: f(integral_constant<int, B>) ... f(integral_constant<int, E - 1>)
@@ -171,6 +174,17 @@ __device__ __forceinline__ void store_row(char *orow, const f32x16 (&acc)[DT], f
         st_global16(orow + dt * 64, oa);
         st_global16(orow + dt * 64 + 16, ob);
     }
+}
+
+// the same as fp32 (partial results that another kernel sums): orow points at element 16*hf of the row
+template <int DT>
+__device__ __forceinline__ void store_row_f32(float *orow, const f32x16 (&acc)[DT], float s) {
+#pragma unroll
+    for (int dt = 0; dt < DT; ++dt)
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4)
+            *reinterpret_cast<float4 *>(orow + 32 * dt + 4 * r4) =
+                make_float4(acc[dt][4 * r4] * s, acc[dt][4 * r4 + 1] * s, acc[dt][4 * r4 + 2] * s, acc[dt][4 * r4 + 3] * s);
 }
 
 // f(integral_constant<int, s mod NS>) for a run-time s (NS = 2, 4 or 8)

@@ -170,7 +170,7 @@ class SlidingTwoSimplicialAttention(Function):
         dk1, dk2, dv1, dv2 = (torch.empty((batch, seq_len, kv_heads, dim), dtype=q.dtype, device=q.device) for _ in range(4))
         prob = _native.problem(batch, seq_len, heads, kv_heads, dim, w1, w2, True, scale)
         # (with the forward's saved partials only the dK2 half of the workspace is used)
-        ws_bytes = lib.sa2_bwd_workspace_bytes(prob) // (2 if t_save is not None else 1)
+        ws_bytes = lib.sa2_bwd_workspace_bytes_with_saved(prob) if t_save is not None else lib.sa2_bwd_workspace_bytes(prob)
         workspace = torch.empty(ws_bytes, dtype=torch.uint8, device=q.device)
         arg = _native.tensor_arg
         with torch.cuda.device_of(q):

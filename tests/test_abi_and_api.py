@@ -80,6 +80,9 @@ def test_argument_validation_happens_before_any_launch(lib):
     need = lib.sa2_bwd_workspace_bytes(good)
     assert need == 2 * 1 * 2 * 2 * 63 * 128 * 4          # 2 tensors, B*H*tiles blocks of 63 fp32 rows
     assert lib.sa2_bwd_workspace_bytes(None) == -1
+    # with saved forward partials: half of the partial rows, but at least the two fp32 partial results of dk1/dv1
+    assert lib.sa2_bwd_workspace_bytes_with_saved(good) == max(need // 2, 2 * 2 * 1 * 1 * 64 * 128 * 4)
+    assert lib.sa2_bwd_workspace_bytes_with_saved(None) == -1
     assert lib.sa2_bwd_dq_dkv2(good, t, t, t, t, t, t, None, lse, None, t, t, t, lse, need, None) == 1
     assert lib.sa2_bwd_dq_dkv2(good, t, t, t, t, t, t, lse, lse, None, t, t, t, None, need, None) == 1
     assert lib.sa2_bwd_dq_dkv2(good, t, t, t, t, t, t, lse, lse, None, t, t, t, lse, need - 1, None) == 2
