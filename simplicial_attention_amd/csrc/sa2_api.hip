@@ -260,11 +260,29 @@ static int64_t partial_rows_bytes(const sa2_problem *prob) {
 }
 
 // dK1/dV1 with the key slabs' work split over two workgroups each (fp32 partial results, summed by a second kernel):
-// for grids that put fewer than four workgroups on a CU, where whole workgroups of unequal length leave many CUs
-// idle at the end.  Depends on the problem only, so that every entry point with a workspace runs the same kernels.
+// for grids of one to four workgroups per CU on short sequences, where the slabs at the sequence's end (those within
+// w1 + 128 rows of it) meet fewer query tiles than the others and whole workgroups of unequal length leave many CUs
+// idle at the end.  Measured on 256 CUs, whole backward: - 3 % and - 8 % at 512 and 896 workgroups of N = 2048, D = 64;
+// - 1 to - 2 % at 512 and 768 of D = 128; + 1 to + 2 % at 256 workgroups and at N = 8192, which the rule leaves alone.
+// It depends on the problem and the device's CU count only, so every entry point with a workspace runs the same kernels.
+static int cu_count() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            cus = n;
+        else
+            cus = 256;
+    }
+    return cus;
+}
+
 static bool dkv1_in_parts(const sa2_problem *prob) {
-    const int64_t grid = (int64_t)prob->batch * prob->kv_heads * ((prob->seq_len + 127) / 128);
-    return grid < 4 * 256;
+    const int ntile = (prob->seq_len + 127) / 128;
+    const int64_t grid = (int64_t)prob->batch * prob->kv_heads * ntile;
+    const int64_t ragged = (prob->w1 + 127) / 128 + 1;          // slabs per sequence with a shortened range of query tiles
+    return grid > cu_count() && grid < 4 * cu_count() && 8 * ragged >= ntile;
 }
 
 static int64_t dkv1_parts_bytes(const sa2_problem *prob) {

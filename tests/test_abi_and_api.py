@@ -80,9 +80,19 @@ def test_argument_validation_happens_before_any_launch(lib):
     need = lib.sa2_bwd_workspace_bytes(good)
     assert need == 2 * 1 * 2 * 2 * 63 * 128 * 4          # 2 tensors, B*H*tiles blocks of 63 fp32 rows
     assert lib.sa2_bwd_workspace_bytes(None) == -1
-    # with saved forward partials: half of the partial rows, but at least the two fp32 partial results of dk1/dv1
-    assert lib.sa2_bwd_workspace_bytes_with_saved(good) == max(need // 2, 2 * 2 * 1 * 1 * 64 * 128 * 4)
+    # with saved forward partials: half of the partial rows ...
+    assert lib.sa2_bwd_workspace_bytes_with_saved(good) == need // 2
     assert lib.sa2_bwd_workspace_bytes_with_saved(None) == -1
+    # ... but at least the two fp32 partial results of dk1/dv1 where the key slabs are split over two workgroups
+    # each (a grid of two ragged workgroups per CU: the layer shape of benchmark config 5 on 256 CUs)
+    layer5 = _native.problem(8, 2048, 8, 4, 64, 512, 32, True, 0.125)
+    rows5 = 2 * 8 * 8 * 64 * 63 * 64 * 4
+    parts5 = 2 * 2 * 8 * 4 * 2048 * 64 * 4
+    assert lib.sa2_bwd_workspace_bytes(layer5) == rows5
+    assert lib.sa2_bwd_workspace_bytes_with_saved(layer5) == max(rows5 // 2, parts5) == parts5
+    # an even grid of equal workgroups is left alone (config 3: eight workgroups per CU)
+    config3 = _native.problem(4, 8192, 8, 8, 128, 512, 32, True, 0.1)
+    assert lib.sa2_bwd_workspace_bytes_with_saved(config3) * 2 == lib.sa2_bwd_workspace_bytes(config3)
     assert lib.sa2_bwd_dq_dkv2(good, t, t, t, t, t, t, None, lse, None, t, t, t, lse, need, None) == 1
     assert lib.sa2_bwd_dq_dkv2(good, t, t, t, t, t, t, lse, lse, None, t, t, t, None, need, None) == 1
     assert lib.sa2_bwd_dq_dkv2(good, t, t, t, t, t, t, lse, lse, None, t, t, t, lse, need - 1, None) == 2

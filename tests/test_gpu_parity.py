@@ -265,18 +265,53 @@ def test_each_backward_entry_point_against_the_oracle():
         row = U.compare(name, got, ref)
         print('  ', row, flush=True)
         assert row['bad'] == 0 and row['rel_fro'] <= 1e-2, row
-    # the whole backward in one call: at this grid size it splits every key slab over two workgroups and sums
-    # their fp32 partial results, so dk1/dv1 may differ from the single-workgroup results by a rounding
+    # the whole backward in one call runs the same kernels (this grid is too small for split key slabs)
     delta2 = torch.empty_like(lse)
     dq2 = torch.full_like(q, float('nan'))
     g2 = [torch.full_like(k1, float('nan')) for _ in range(4)]
     _native.check(lib.sa2_bwd(prob, arg(q), arg(k1), arg(k2), arg(v1), arg(v2), arg(out), arg(res), arg(dout), lse.data_ptr(), None,
                               delta2.data_ptr(), arg(dq2), arg(g2[0]), arg(g2[1]), arg(g2[2]), arg(g2[3]), ws.data_ptr(), ws_bytes, sh))
     torch.cuda.synchronize()
-    for name, got, one, ref in (('dk1', g2[0], dk1, ref_grads[1]), ('dv1', g2[2], dv1, ref_grads[3])):
-        row = U.compare(name, got, ref)
-        print('  in parts', row, flush=True)
-        assert row['bad'] == 0 and row['rel_fro'] <= 1e-2, row
-        diff = (got.float() - one.float()).abs()
-        assert float((diff / one.float().abs().clamp_min(1e-3)).max()) <= 2 ** -7, name     # one bf16 rounding
     assert torch.equal(dq2, dq) and torch.equal(g2[1], dk2) and torch.equal(g2[3], dv2)
+    assert torch.equal(g2[0], dk1) and torch.equal(g2[2], dv1)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize('d', [32, 128])
+def test_split_key_slabs_against_the_oracle_and_single_workgroups(d):
+    """A grid of one to four dK1/dV1 workgroups per CU on a short sequence: sa2_bwd gives every key slab to two
+    workgroups (half of the slab's query tiles each) and adds their fp32 partial results; sa2_bwd_dkv1, which has
+    no workspace, keeps one workgroup per slab.  Both against the oracle, and against each other to one rounding."""
+    from simplicial_attention_amd import _native
+    lib = _native.load()
+    arg = _native.tensor_arg
+    b, n, hq, hk, w1, w2 = 3, 1024, 12, 12, 64, 8
+    prob = _native.problem(b, n, hq, hk, d, w1, w2, True, d ** -0.5)
+    parts = 2 * 2 * b * hk * n * d * 4
+    if lib.sa2_bwd_workspace_bytes_with_saved(prob) != parts:
+        pytest.skip('this device has too many CUs for the split to apply at this size')
+    ins = U.make_inputs(b, n, hq, hk, d, seed=5, std=d ** -0.5)
+    _, _, ref_grads = U.oracle_fwd_bwd(*ins, w1, w2)
+    q, k1, k2, v1, v2, dout = (t.cuda() for t in ins)
+    sh = torch.cuda.current_stream().cuda_stream
+    out, res = torch.empty_like(q), torch.empty_like(q)
+    lse = torch.empty(b, hq, n, dtype=torch.float32, device='cuda')
+    _native.check(lib.sa2_fwd(prob, arg(q), arg(k1), arg(k2), arg(v1), arg(v2), arg(out), arg(res), lse.data_ptr(), None, sh))
+    delta = torch.empty_like(lse)
+    ws_bytes = lib.sa2_bwd_workspace_bytes(prob)
+    ws = torch.empty(ws_bytes, dtype=torch.uint8, device='cuda')
+    dq = torch.full_like(q, float('nan'))
+    g = [torch.full_like(k1, float('nan')) for _ in range(4)]
+    _native.check(lib.sa2_bwd(prob, arg(q), arg(k1), arg(k2), arg(v1), arg(v2), arg(out), arg(res), arg(dout), lse.data_ptr(), None,
+                              delta.data_ptr(), arg(dq), arg(g[0]), arg(g[1]), arg(g[2]), arg(g[3]), ws.data_ptr(), ws_bytes, sh))
+    one = [torch.full_like(k1, float('nan')) for _ in range(2)]
+    _native.check(lib.sa2_bwd_dkv1(prob, arg(q), arg(k1), arg(k2), arg(v1), arg(v2), arg(dout), lse.data_ptr(), delta.data_ptr(),
+                                   arg(one[0]), arg(one[1]), sh))
+    torch.cuda.synchronize()
+    for name, got, single, ref in (('dk1', g[0], one[0], ref_grads[1]), ('dv1', g[2], one[1], ref_grads[3])):
+        for label, t in (('in parts', got), ('single', single)):
+            row = U.compare(name, t, ref)
+            print('  ', label, row, flush=True)
+            assert row['bad'] == 0 and row['rel_fro'] <= 1e-2, (label, row)
+        diff = (got.float() - single.float()).abs()
+        assert float((diff / single.float().abs().clamp_min(1e-3)).max()) <= 2 ** -7, name     # one bf16 rounding
