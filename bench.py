@@ -130,7 +130,8 @@ def kernel_symbol(entry, D, w2):
     if entry == 'bwd_dq_dk2_pass':
         return 'sa2::bwd_q_kernel<%d, true>' % D
     if entry == 'bwd_dkv1':
-        return 'sa2::bwd_kv8_kernel<%d, %d>' % (D, 3 if D == 128 else 2)
+        # (the entry point sa2_bwd_dkv1 has no workspace and always runs one workgroup per key slab: PARTS = false)
+        return 'sa2::bwd_kv8_kernel<%d, %d, false>' % (D, 3 if D == 128 else 2)
     return None
 
 
@@ -194,6 +195,126 @@ def traffic_from(directory):
     json.dump(rec, open(TRAFFIC_FILE, 'w'), indent=1, sort_keys=True)
     print(json.dumps(rec))
 
+def time_raw_workload(name, steps=5, warmup=2):
+    """forward + backward of the raw kernel path at workload `name` through the autograd Function: ms per step,
+    TFLOP/s on the 18*D*B*H*P count and the fraction of the bf16 MFMA peak."""
+    import torch
+    from simplicial_attention_amd import sliding_two_simplicial_attn
+    B, H, HK, N, D, w1, w2 = WORKLOADS[name]
+    dev = torch.device('cuda:0')
+    g = torch.Generator(device='cpu').manual_seed(3)
+    mk = lambda h, sc: (torch.randn(B, N, h, D, generator=g) * sc).bfloat16().to(dev)
+    ins = [mk(H, D ** -0.5)] + [mk(HK, D ** -0.5) for _ in range(4)]
+    dout = mk(H, 1.0)
+    ins = [t.requires_grad_(True) for t in ins]
+
+    def step():
+        out = sliding_two_simplicial_attn(ins[0], (ins[1], ins[2]), (ins[3], ins[4]), w1=w1, w2=w2, causal=True)
+        return torch.autograd.grad(out, ins, dout)
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    t = (time.perf_counter() - t0) / steps
+    flops = 18 * D * B * H * attended_triples(N, w1, w2)
+    del ins, dout
+    torch.cuda.empty_cache()
+    return {'ms_per_step': round(t * 1e3, 3), 'tflops': round(flops / t / 1e12, 2),
+            'frac_of_bf16_peak': round(flops / t / 1e12 / PEAK_BF16_TFLOPS, 4), 'tokens_per_s': round(B * N / t, 1), 'steps': steps}
+
+
+def time_train_cfg5(steps=5, warmup=2):
+    """benchmark config 5: one training step (forward, loss, backward, Adam) of the byte-level LM: depth 12, dim 512,
+    8 heads of 64 (4 key/value heads), every 2nd layer simplicial (w1=512, w2=32), batch 8 x 2048 random bytes; and the
+    share of the six simplicial attention cores (the same Function at the layer's shape, timed alone)."""
+    import torch
+    from simplicial_attention_amd import sliding_two_simplicial_attn
+    from simplicial_attention_amd.two_simplicial_transformer import TwoSimplicialLM
+    dev = torch.device('cuda:0')
+    torch.manual_seed(4)
+    lm = TwoSimplicialLM(num_tokens=256, dim=512, depth=12, max_seq_len=2048, dim_head=64, heads=8,
+                         two_simplicial_attn_every=2, transformer_kwargs=dict(key_value_heads=4)).bfloat16().to(dev)
+    opt = torch.optim.Adam(lm.parameters(), lr=1e-4)
+    tokens = torch.randint(0, 256, (8, 2049), device=dev)
+
+    def train_step():
+        opt.zero_grad(set_to_none=True)
+        loss = lm(tokens, return_loss=True)
+        loss.backward()
+        opt.step()
+        return loss
+    for _ in range(max(2, warmup)):
+        train_step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        loss = train_step()
+    torch.cuda.synchronize()
+    step_ms = (time.perf_counter() - t0) / steps * 1e3
+    mk5 = lambda h: (torch.randn(8, 2048, h, 64, device=dev) * 0.125).bfloat16().requires_grad_(True)
+    q5, k15, k25, v15, v25 = mk5(8), mk5(4), mk5(4), mk5(4), mk5(4)
+    do5 = torch.randn(8, 2048, 8, 64, device=dev).bfloat16()
+
+    def core():
+        o = sliding_two_simplicial_attn(q5, (k15, k25), (v15, v25), w1=512, w2=32)
+        torch.autograd.grad(o, (q5, k15, k25, v15, v25), do5)
+    for _ in range(3):
+        core()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(10):
+        core()
+    torch.cuda.synchronize()
+    core_ms = (time.perf_counter() - t0) / 10 * 1e3
+    res = {'workload': 'cfg5_training_step_depth12_dim512_b8_n2048', 'ms_per_step': round(step_ms, 3),
+           'tokens_per_s': round(8 * 2048 / step_ms * 1e3, 1), 'loss': round(loss.item(), 4),
+           'simplicial_core_fwd_bwd_ms_per_layer': round(core_ms, 3),
+           'simplicial_cores_share_of_step': round(6 * core_ms / step_ms, 3), 'steps': steps}
+    del lm, opt
+    torch.cuda.empty_cache()
+    return res
+
+
+def time_module_cfg2(iters=50):
+    """benchmark config 2: the multi-head module, tokens (2, 1024, 512), dim_head 64, 8 heads, forward, with and
+    without the fused split + RMSNorm kernel; and that kernel alone at the config-3 token count."""
+    import torch
+    from simplicial_attention_amd import SlidingWindowTwoSimplicialMHA
+    from simplicial_attention_amd.qkv_norm import FusedQKVNorm
+    dev = torch.device('cuda:0')
+    torch.manual_seed(1)
+    m = SlidingWindowTwoSimplicialMHA(512, dim_head=64, heads=8, w1=512, w2=32).bfloat16().to(dev)
+    tokens = torch.randn(2, 1024, 512, device=dev).bfloat16()
+
+    def timed(fn, n):
+        for _ in range(5):
+            fn()
+        torch.cuda.synchronize()
+        a, b_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(n):
+            fn()
+        b_.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b_) / n
+    res = {}
+    with torch.no_grad():
+        for fused in (True, False):
+            m.fused_qkv_norm = fused
+            res['module_fwd_ms_fused' if fused else 'module_fwd_ms_unfused'] = round(timed(lambda: m(tokens), iters), 4)
+        bq, nq, hq, dq_ = 4, 8192, 8, 128
+        qkv = torch.randn(bq, nq, 5 * hq * dq_, device=dev).bfloat16()
+        w = torch.ones(dq_, device=dev).bfloat16()
+        ms = timed(lambda: FusedQKVNorm.apply(qkv, w, w, w, w, w, hq, hq, dq_, 1e-6), 20)
+        nbytes = 2 * qkv.numel() * 2 + 4 * bq * nq * 5 * hq
+        res['qkv_norm_fwd'] = {'tokens': bq * nq, 'channels': 5 * hq * dq_, 'ms': round(ms, 4),
+                               'hbm_bytes': nbytes, 'achieved_gbs': round(nbytes / ms / 1e6, 1), 'peak_gbs': PEAK_HBM_GBS}
+    res['tokens_per_s'] = round(2 * 1024 / res['module_fwd_ms_fused'] * 1e3, 1)
+    return res
+
 
 def main():
     ap = argparse.ArgumentParser()
@@ -203,6 +324,8 @@ def main():
     ap.add_argument('--workload', default='cfg3_raw_kernel_b4_h8_n8192_d128_w512_w32', choices=sorted(WORKLOADS))
     ap.add_argument('--cpu-slices', type=int, default=4, help='(batch, head) slices of the CPU baseline sample (0 = skip)')
     ap.add_argument('--kernel-iters', type=int, default=5, help='launches per kernel for the per-kernel timing')
+    ap.add_argument('--no-other-workloads', dest='other_workloads', action='store_false',
+                    help='skip the other benchmark workloads (config 4, the config-5 layer and training step, the config-2 module) that the default run times after config 3')
     ap.add_argument('--traffic-from', default=None, metavar='DIR', help='no GPU work: read the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE passes under DIR and write profiles/hbm_traffic.json')
     ap.add_argument('--only', default=None, help='time only this entry through the C ABI (fwd, bwd_delta, bwd_dq_dkv2, bwd_dkv1, bwd_dq_dk2_pass), `copy`: a 1 GiB device copy that calibrates HBM counters; `module_cfg2`: the module forward of config 2 and the fused qkv-norm kernel; `train_cfg5`: one training step of the config-5 language model; for profiling')
     args = ap.parse_args()
@@ -226,83 +349,10 @@ def main():
     B, H, HK, N, D, w1, w2 = WORKLOADS[args.workload]
     dev = torch.device('cuda:0')
     if args.only == 'train_cfg5':
-        # benchmark config 5: one training step (forward, loss, backward, Adam) of the byte-level LM: depth 12,
-        # dim 512, 8 heads of 64 (4 key/value heads), every 2nd layer simplicial (w1=512, w2=32), batch 8 x 2048
-        from simplicial_attention_amd.two_simplicial_transformer import TwoSimplicialLM
-        torch.manual_seed(4)
-        lm = TwoSimplicialLM(num_tokens=256, dim=512, depth=12, max_seq_len=2048, dim_head=64, heads=8,
-                             two_simplicial_attn_every=2, transformer_kwargs=dict(key_value_heads=4)).bfloat16().to(dev)
-        opt = torch.optim.Adam(lm.parameters(), lr=1e-4)
-        tokens = torch.randint(0, 256, (8, 2049), device=dev)
-
-        def train_step():
-            opt.zero_grad(set_to_none=True)
-            loss = lm(tokens, return_loss=True)
-            loss.backward()
-            opt.step()
-            return loss
-        for _ in range(max(2, args.warmup)):
-            train_step()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            loss = train_step()
-        torch.cuda.synchronize()
-        step_ms = (time.perf_counter() - t0) / args.steps * 1e3
-        # share of the six simplicial attention cores: the same Function at the layer's shape, timed alone
-        mk5 = lambda h: (torch.randn(8, 2048, h, 64, device=dev) * 0.125).bfloat16().requires_grad_(True)
-        q5, k15, k25, v15, v25 = mk5(8), mk5(4), mk5(4), mk5(4), mk5(4)
-        do5 = torch.randn(8, 2048, 8, 64, device=dev).bfloat16()
-
-        def core():
-            o = sliding_two_simplicial_attn(q5, (k15, k25), (v15, v25), w1=512, w2=32)
-            torch.autograd.grad(o, (q5, k15, k25, v15, v25), do5)
-        for _ in range(3):
-            core()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(10):
-            core()
-        torch.cuda.synchronize()
-        core_ms = (time.perf_counter() - t0) / 10 * 1e3
-        print(json.dumps({'workload': 'cfg5_training_step_depth12_dim512_b8_n2048', 'ms_per_step': round(step_ms, 3),
-                          'tokens_per_s': round(8 * 2048 / step_ms * 1e3, 1), 'loss': round(loss.item(), 4),
-                          'simplicial_core_fwd_bwd_ms_per_layer': round(core_ms, 3),
-                          'simplicial_cores_share_of_step': round(6 * core_ms / step_ms, 3), 'steps': args.steps}))
+        print(json.dumps(time_train_cfg5(args.steps, args.warmup)))
         return
     if args.only == 'module_cfg2':
-        # benchmark config 2: the multi-head module, tokens (2, 1024, 512), dim_head 64, 8 heads, forward,
-        # with and without the fused split + RMSNorm kernel; and that kernel alone at the config-3 token count
-        from simplicial_attention_amd import SlidingWindowTwoSimplicialMHA
-        from simplicial_attention_amd.qkv_norm import FusedQKVNorm
-        torch.manual_seed(1)
-        m = SlidingWindowTwoSimplicialMHA(512, dim_head=64, heads=8, w1=512, w2=32).bfloat16().to(dev)
-        tokens = torch.randn(2, 1024, 512, device=dev).bfloat16()
-
-        def timed(fn, iters=50):
-            for _ in range(5):
-                fn()
-            torch.cuda.synchronize()
-            a, b_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-            a.record()
-            for _ in range(iters):
-                fn()
-            b_.record()
-            torch.cuda.synchronize()
-            return a.elapsed_time(b_) / iters
-        res = {}
-        with torch.no_grad():
-            for fused in (True, False):
-                m.fused_qkv_norm = fused
-                res['module_fwd_ms_fused' if fused else 'module_fwd_ms_unfused'] = round(timed(lambda: m(tokens)), 4)
-            bq, nq, hq, dq_ = 4, 8192, 8, 128
-            qkv = torch.randn(bq, nq, 5 * hq * dq_, device=dev).bfloat16()
-            w = torch.ones(dq_, device=dev).bfloat16()
-            ms = timed(lambda: FusedQKVNorm.apply(qkv, w, w, w, w, w, hq, hq, dq_, 1e-6), 20)
-            nbytes = 2 * qkv.numel() * 2 + 4 * bq * nq * 5 * hq
-            res['qkv_norm_fwd'] = {'tokens': bq * nq, 'channels': 5 * hq * dq_, 'ms': round(ms, 4),
-                                   'hbm_bytes': nbytes, 'achieved_gbs': round(nbytes / ms / 1e6, 1), 'peak_gbs': PEAK_HBM_GBS}
-        print(json.dumps(res))
+        print(json.dumps(time_module_cfg2()))
         return
     if args.only == 'copy':
         # plain device copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters
@@ -426,9 +476,32 @@ def main():
     dom = max(single, key=lambda k: kernels[k]['ms'])
     achieved = kernels[dom]['tflops']
     traffic, traffic_note = stored_traffic(args.workload, dom)
+    # the dominant kernel inside the step: the whole backward through sa2_bwd (HIP events on the launch stream) minus
+    # the stand-alone times of its other entries
+    in_step_ms = None
+    if dom == 'bwd_dkv1':
+        g5 = [torch.empty_like(qd)] + [torch.empty_like(k1d) for _ in range(4)]
+        bwd_all = lambda: lib.sa2_bwd(prob, *five, arg(out), arg(res), arg(dout), lse.data_ptr(), saved, delta.data_ptr(),
+                                      arg(g5[0]), arg(g5[1]), arg(g5[2]), arg(g5[3]), arg(g5[4]), ws.data_ptr(), ws_bytes, sh)
+        _native.check(bwd_all())
+        torch.cuda.synchronize()
+        evs = []
+        for _ in range(args.kernel_iters):
+            a, b_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            a.record(stream)
+            _native.check(bwd_all())
+            b_.record(stream)
+            evs.append((a, b_))
+        torch.cuda.synchronize()
+        bwd_ms = statistics.mean(a.elapsed_time(b_) for a, b_ in evs)
+        kernels['bwd_whole'] = {'ms': round(bwd_ms, 4), 'contractions': 7, 'tflops': round(7 * unit / (bwd_ms * 1e-3) / 1e12, 2)}
+        in_step_ms = round(bwd_ms - kernels['bwd_delta']['ms'] - kernels['bwd_dq_dkv2']['ms'], 4)
     roofline = {'bound': 'mfma', 'kernel': dom, 'kernel_symbol': kernel_symbol(dom, D, w2), 'achieved': achieved, 'peak': PEAK_BF16_TFLOPS, 'unit': 'TFLOP/s',
                 'frac': round(achieved / PEAK_BF16_TFLOPS, 4), 'traffic': traffic, 'traffic_note': traffic_note,
                 'launch_ms': kernels[dom]['ms'],
+                'in_step_ms': in_step_ms,
+                'frac_in_step': round(kernels[dom]['contractions'] * unit / (in_step_ms * 1e-3) / 1e12 / PEAK_BF16_TFLOPS, 4) if in_step_ms else None,
+                'in_step_note': 'launch_ms: the kernel alone in a loop; in_step_ms: the whole backward (sa2_bwd) minus its other entries timed alone',
                 'flops_per_launch': kernels[dom]['contractions'] * unit}
 
     total_flops = 9 * unit          # 18*D*B*H*P
@@ -449,6 +522,15 @@ def main():
         'kernels': kernels,
         'roofline': roofline,
     }
+    if args.other_workloads and args.workload == 'cfg3_raw_kernel_b4_h8_n8192_d128_w512_w32':
+        # the other benchmark workloads, timed in the same run (each at least 5 steps)
+        torch.cuda.empty_cache()
+        other = {}
+        for name in ('cfg4_long_context_b1_h16_n32768_d128_w512_w32', 'cfg5_layer_b8_h8_kv4_n2048_d64_w512_w32'):
+            other[name] = time_raw_workload(name, steps=5 if 'cfg4' in name else 10)
+        other['cfg5_training_step_depth12_dim512_b8_n2048'] = time_train_cfg5(steps=5)
+        other['cfg2_module_forward_b2_n1024_dim512'] = time_module_cfg2(iters=20)
+        result['other_workloads'] = other
     if args.cpu_slices > 0:
         result['cpu_baseline'] = cpu_baseline(N, D, w1, w2, args.cpu_slices)
     print(json.dumps(result))

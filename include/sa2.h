@@ -22,9 +22,11 @@
  *     (triton_two_simplicial_attention.py:191-193).  Only causal = 1 is defined.
  *   - seq_len is arbitrary: rows past the end are masked in-kernel, so the caller
  *     does not need the zero padding of triton_two_simplicial_attention.py:1042-1046.
- *   - All calls are asynchronous on the given stream, allocate nothing, keep no
- *     device state and may be issued from any host thread.  Buffers are owned by
- *     the caller.  The device is the caller's current HIP device.
+ *   - All calls are asynchronous on the given stream, allocate nothing and may be
+ *     issued from any host thread.  Buffers are owned by the caller, and the library
+ *     keeps no device state - except sa2_bwd_noalloc, whose scratch is a fixed
+ *     device array inside the library (see there).  The device is the caller's
+ *     current HIP device.
  *   - Return value: SA2_OK or an sa2_status; sa2_last_error() gives a
  *     thread-local message for the last failure on the calling thread.
  */
@@ -37,7 +39,9 @@
 extern "C" {
 #endif
 
-#define SA2_VERSION 100
+/* 101: saved->t is kept in blocks of 32 rows (sa2_saved_t_bytes), the workspace rules of sa2_bwd_workspace_bytes*
+ * cover the split key slabs, sa2_bwd checks every size before its first launch */
+#define SA2_VERSION 101
 
 typedef enum sa2_status {
     SA2_OK = 0,

@@ -262,21 +262,12 @@ static int64_t partial_rows_bytes(const sa2_problem *prob) {
 // dK1/dV1 with the key slabs' work split over two workgroups each (fp32 partial results, summed by a second kernel):
 // for grids of one to four workgroups per CU on short sequences, where the slabs at the sequence's end (those within
 // w1 + 128 rows of it) meet fewer query tiles than the others and whole workgroups of unequal length leave many CUs
-// idle at the end.  Measured on 256 CUs, whole backward: - 3 % and - 8 % at 512 and 896 workgroups of N = 2048, D = 64;
-// - 1 to - 2 % at 512 and 768 of D = 128; + 1 to + 2 % at 256 workgroups and at N = 8192, which the rule leaves alone.
-// It depends on the problem and the device's CU count only, so every entry point with a workspace runs the same kernels.
-static int cu_count() {
-    static int cus = 0;
-    if (cus == 0) {
-        int dev = 0, n = 0;
-        if (hipGetDevice(&dev) == hipSuccess &&
-            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
-            cus = n;
-        else
-            cus = 256;
-    }
-    return cus;
-}
+// idle at the end.  Measured on the 256 CUs of an MI355X, whole backward: - 3 % and - 8 % at 512 and 896 workgroups of
+// N = 2048, D = 64; - 1 to - 2 % at 512 and 768 of D = 128; + 1 to + 2 % at 256 workgroups and at N = 8192, which the rule
+// leaves alone.  The rule is a function of the problem alone (the library is built for this one chip), so workspace sizes
+// and the kernels that run do not depend on the device or on which thread asked first.
+static constexpr int kComputeUnits = 256;
+static int cu_count() { return kComputeUnits; }
 
 static bool dkv1_in_parts(const sa2_problem *prob) {
     const int ntile = (prob->seq_len + 127) / 128;
@@ -302,11 +293,21 @@ int64_t sa2_bwd_workspace_bytes_with_saved(const sa2_problem *prob) {
     return max64(partial_rows_bytes(prob) / 2, dkv1_parts_bytes(prob));
 }
 
-int sa2_bwd_dq_dkv2(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
-                    const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *dout, const float *lse,
-                    const float *delta, const sa2_saved *saved, const sa2_tensor *dq, const sa2_tensor *dk2,
-                    const sa2_tensor *dv2, void *workspace, int64_t workspace_bytes, void *hip_stream) {
+// The launches behind sa2_bwd_dq_dkv2: the MFMA kernel(s) on stream `s`; the kernel that streams the forward's saved
+// partials on `s_dv2` (it depends on nothing the backward computes); the reduction of the partial rows on `s_comb`
+// (it follows the MFMA kernel: the caller orders the streams).
+struct QLaunch {
     sa2::KParams k;
+    float *ws;
+    int grid, halo;
+    bool use_saved;
+};
+
+static int prepare_dq_dkv2(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
+                           const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *dout, const float *lse,
+                           const float *delta, const sa2_saved *saved, const sa2_tensor *dq, const sa2_tensor *dk2,
+                           const sa2_tensor *dv2, void *workspace, int64_t workspace_bytes, QLaunch *out) {
+    sa2::KParams &k = out->k;
     SA2_TRY(bwd_common(prob, q, k1, k2, v1, v2, dout, lse, delta, &k));
     SA2_TRY(check_tensor(dq, "dq"));
     SA2_TRY(check_tensor(dk2, "dk2"));
@@ -323,35 +324,54 @@ int sa2_bwd_dq_dkv2(const sa2_problem *prob, const sa2_tensor *q, const sa2_tens
     k.dq = dev(dq);
     k.dk2 = dev(dk2);
     k.dv2 = dev(dv2);
-    float *ws = static_cast<float *>(workspace);
-    hipStream_t s = static_cast<hipStream_t>(hip_stream);
-    const int grid = prob->batch * prob->heads * ((prob->seq_len + 31) / 32);
-    const int halo = q_halo(prob->w2);
-    const int pass = bwd_pass_filter();
+    out->ws = static_cast<float *>(workspace);
+    out->grid = prob->batch * prob->heads * ((prob->seq_len + 31) / 32);
+    out->halo = q_halo(prob->w2);
     // with the forward's saved per-offset T the dv2 pass (a recomputation of S and T) is
     // replaced by a kernel that streams T once
-    const bool use_saved = saved != nullptr;
+    out->use_saved = saved_given;
     if (saved) {
         SA2_TRY(check_saved(saved));
         k.t_save = static_cast<char *>(saved->t);
         k.m_save = saved->m;
     }
-    SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL((sa2::bwd_q_kernel<DH, true>), dim3(grid), dim3(512), 0, s, k, ws, halo));
-    if (pass != 1 && !use_saved)
-        SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL((sa2::bwd_q_kernel<DH, false>), dim3(grid), dim3(512), 0, s, k, ws, halo));
-    SA2_TRY(after_launch("dq/dk2/dv2"));
-    if (pass == 1) return SA2_OK;    // profiling build, one pass: leave the reductions out of its timing
-    if (use_saved) {
-        const int dgrid = prob->batch * prob->kv_heads * ((prob->seq_len + 31) / 32);
-        SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL(sa2::dv2_from_saved_kernel<DH>, dim3(dgrid), dim3(sa2::Dv2Cfg<DH>::THREADS), 0, s, k));
-        SA2_TRY(after_launch("dv2 from saved partials"));
-    }
+    return SA2_OK;
+}
+
+static int launch_q_mfma(const sa2_problem *prob, const QLaunch &L, int pass, hipStream_t s) {
+    SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL((sa2::bwd_q_kernel<DH, true>), dim3(L.grid), dim3(512), 0, s, L.k, L.ws, L.halo));
+    if (pass != 1 && !L.use_saved)
+        SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL((sa2::bwd_q_kernel<DH, false>), dim3(L.grid), dim3(512), 0, s, L.k, L.ws, L.halo));
+    return after_launch("dq/dk2/dv2");
+}
+
+static int launch_dv2_from_saved(const sa2_problem *prob, const QLaunch &L, hipStream_t s) {
+    const int dgrid = prob->batch * prob->kv_heads * ((prob->seq_len + 31) / 32);
+    SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL(sa2::dv2_from_saved_kernel<DH>, dim3(dgrid), dim3(sa2::Dv2Cfg<DH>::THREADS), 0, s, L.k));
+    return after_launch("dv2 from saved partials");
+}
+
+static int launch_q_combine(const sa2_problem *prob, const QLaunch &L, hipStream_t s) {
     const int64_t rows = (int64_t)prob->batch * prob->kv_heads * prob->seq_len;
     const int rows_per_block = 256 / (prob->dim_head / 8);
     const int cgrid = (int)((rows + rows_per_block - 1) / rows_per_block);
-    const int with_dv2 = use_saved ? 0 : 1;
-    SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL(sa2::dk2_dv2_combine_kernel<DH>, dim3(cgrid), dim3(256), 0, s, k, ws, 32 + halo, with_dv2));
+    const int with_dv2 = L.use_saved ? 0 : 1;
+    SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL(sa2::dk2_dv2_combine_kernel<DH>, dim3(cgrid), dim3(256), 0, s, L.k, L.ws, 32 + L.halo, with_dv2));
     return after_launch("dk2/dv2 combine");
+}
+
+int sa2_bwd_dq_dkv2(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
+                    const sa2_tensor *v1, const sa2_tensor *v2, const sa2_tensor *dout, const float *lse,
+                    const float *delta, const sa2_saved *saved, const sa2_tensor *dq, const sa2_tensor *dk2,
+                    const sa2_tensor *dv2, void *workspace, int64_t workspace_bytes, void *hip_stream) {
+    QLaunch L;
+    SA2_TRY(prepare_dq_dkv2(prob, q, k1, k2, v1, v2, dout, lse, delta, saved, dq, dk2, dv2, workspace, workspace_bytes, &L));
+    hipStream_t s = static_cast<hipStream_t>(hip_stream);
+    const int pass = bwd_pass_filter();
+    SA2_TRY(launch_q_mfma(prob, L, pass, s));
+    if (pass == 1) return SA2_OK;    // profiling build, one pass: leave the reductions out of its timing
+    if (L.use_saved) SA2_TRY(launch_dv2_from_saved(prob, L, s));
+    return launch_q_combine(prob, L, s);
 }
 
 static int launch_dkv1(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, const sa2_tensor *k2,
@@ -401,17 +421,26 @@ int sa2_bwd(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, 
             const sa2_tensor *dout, const float *lse, const sa2_saved *saved, float *delta_ws, const sa2_tensor *dq,
             const sa2_tensor *dk1, const sa2_tensor *dk2, const sa2_tensor *dv1, const sa2_tensor *dv2, void *workspace,
             int64_t workspace_bytes, void *hip_stream) {
+    SA2_TRY(check_problem(prob));
+    // every size and pointer is checked before the first launch: a call that fails has written nothing
+    const bool parts_wanted = dkv1_in_parts(prob);
+    if (parts_wanted && workspace_bytes < dkv1_parts_bytes(prob))
+        return fail(SA2_ERR_BAD_SHAPE, "workspace of %lld bytes is smaller than the %lld bytes this problem's dk1/dv1 pass needs (sa2_bwd_workspace_bytes())",
+                    (long long)workspace_bytes, (long long)dkv1_parts_bytes(prob));
+    if (!delta_ws) return fail(SA2_ERR_NULL_POINTER, "delta is NULL");
+    SA2_TRY(check_tensor(out, "out"));
+    if (out_residual) SA2_TRY(check_tensor(out_residual, "out_residual"));
+    SA2_TRY(check_tensor(dk1, "dk1"));
+    SA2_TRY(check_tensor(dv1, "dv1"));
+    QLaunch L;
+    SA2_TRY(prepare_dq_dkv2(prob, q, k1, k2, v1, v2, dout, lse, delta_ws, saved, dq, dk2, dv2, workspace, workspace_bytes, &L));
+    hipStream_t s = static_cast<hipStream_t>(hip_stream);
     SA2_TRY(sa2_bwd_delta(prob, out, out_residual, dout, delta_ws, hip_stream));
-    SA2_TRY(sa2_bwd_dq_dkv2(prob, q, k1, k2, v1, v2, dout, lse, delta_ws, saved, dq, dk2, dv2, workspace,
-                            workspace_bytes, hip_stream));
+    SA2_TRY(launch_q_mfma(prob, L, 0, s));
+    if (L.use_saved) SA2_TRY(launch_dv2_from_saved(prob, L, s));
+    SA2_TRY(launch_q_combine(prob, L, s));
     // the partial rows of dK2/dV2 are spent by now: the partial results of split key slabs reuse the workspace
-    float *parts = nullptr;
-    if (dkv1_in_parts(prob)) {
-        if (workspace_bytes < dkv1_parts_bytes(prob))
-            return fail(SA2_ERR_BAD_SHAPE, "workspace of %lld bytes is smaller than the %lld bytes this problem's dk1/dv1 pass needs (sa2_bwd_workspace_bytes())",
-                        (long long)workspace_bytes, (long long)dkv1_parts_bytes(prob));
-        parts = static_cast<float *>(workspace);
-    }
+    float *parts = parts_wanted ? static_cast<float *>(workspace) : nullptr;
     return launch_dkv1(prob, q, k1, k2, v1, v2, dout, lse, delta_ws, dk1, dv1, parts, hip_stream);
 }
 

@@ -26,7 +26,6 @@
 //                  are issued behind the eight MFMAs of a chain that does not depend on them.
 //                  The P waves build three quarters of the tiles, the S waves one (the S waves
 //                  are the busier ones behind the barrier).
-// (MODEs kKvDk / kKvDv, the two-pass forms that each recompute S, are not instantiated.)
 // Every MFMA chain requests its LDS fragments three places ahead (mfma_stream).
 // S and dP read row fragments of the A and B tiles (ds_read_b128), the accumulating
 // products read transposed fragments (ds_read_b64_tr_b16).  A tile that is read both ways
@@ -40,27 +39,16 @@
 
 namespace sa2 {
 
-constexpr int kKvDv = 0, kKvDk = 1, kKvBoth = 2, kKvSplit = 3;
+constexpr int kKvBoth = 2, kKvSplit = 3;
 
 template <int D, int MODE>
 struct Kv8Cfg {
-    static_assert(MODE == kKvBoth || MODE == kKvSplit, "only the single-kernel forms are built");
-    static constexpr bool DK = MODE != kKvDv;         // dK1 is produced (needs dP, delta, V1)
-    static constexpr bool DV = MODE != kKvDk;         // dV1 is produced
-    static constexpr int PITCH = tile_pitch<D>();
-    static constexpr int TILE = 32 * PITCH;
+    static_assert(MODE == kKvBoth || MODE == kKvSplit, "the two forms of the kernel");
     static constexpr int TPITCH = tr_pitch<D>();
-    static constexpr int TRT = 32 * TPITCH;
-    // step buffer: dk1:  [A swizzled][B row-major][lse][delta]
-    //              dv1:  [A row-major][B transposed-read][lse]
-    //              both: [A swizzled][B swizzled][lse][delta]
-    static constexpr bool A_SWZ = DK;                 // A is read both ways
-    static constexpr bool B_SWZ = DK && DV;           // B is read both ways
-    static constexpr int A_PITCH = A_SWZ ? TPITCH : PITCH;
-    static constexpr int B_PITCH = DV ? TPITCH : PITCH;
+    // step buffer: [A swizzled][B swizzled][lse][delta]  (both tiles are read both ways: see sa2_lds.hpp)
     static constexpr int AS = 0;
-    static constexpr int BS = 32 * A_PITCH;
-    static constexpr int LSE = BS + 32 * B_PITCH;
+    static constexpr int BS = 32 * TPITCH;
+    static constexpr int LSE = BS + 32 * TPITCH;
     static constexpr int DEL = LSE + 32 * 4;
     static constexpr int STEP = DEL + 32 * 4;
     static constexpr int PAIR = 2 * STEP;
@@ -90,9 +78,8 @@ template <int D, int MODE, bool PARTS = false>
 __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     constexpr int KS = D / 16, DT = D / 32, PPR = D / 8;
     using L = Kv8Cfg<D, MODE>;
-    constexpr bool DK = L::DK, TWO = MODE == kKvBoth, SPLIT = MODE == kKvSplit;
+    constexpr bool TWO = MODE == kKvBoth, SPLIT = MODE == kKvSplit;
     static_assert(!TWO || D <= 64, "both accumulators fit two waves per SIMD up to D = 64 only");
-    constexpr int PITCH = L::PITCH;
     __shared__ __attribute__((aligned(16))) char lds[L::LDS];
 
     const int N = p.N;
@@ -118,7 +105,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     const char *v2g = p.v2.ptr + b * p.v2.sb + hk * p.v2.sh;
 
     u32x4 k1f[KS];                        // kKvSplit: the K1 rows in the P waves, the V1 rows in the S waves
-    u32x4 v1f[(DK && !SPLIT) ? KS : 1];
+    u32x4 v1f[SPLIT ? 1 : KS];
     {
         const char *k1row = p.k1.ptr + b * p.k1.sb + (int64_t)jc * p.k1.sn + hk * p.k1.sh;
         const char *v1row = p.v1.ptr + b * p.v1.sb + (int64_t)jc * p.v1.sn + hk * p.v1.sh;
@@ -126,11 +113,11 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
 #pragma unroll
         for (int kk = 0; kk < KS; ++kk) {
             k1f[kk] = ld_global16(own + (16 * kk + 8 * hf) * 2);
-            if constexpr (DK && !SPLIT) v1f[kk] = ld_global16(v1row + (16 * kk + 8 * hf) * 2);
+            if constexpr (!SPLIT) v1f[kk] = ld_global16(v1row + (16 * kk + 8 * hf) * 2);
         }
     }
-    f32x16 acc[DT];              // dK1 (dV1 in the dv1-only pass)
-    f32x16 acc2[TWO ? DT : 1];   // dV1 when both are produced
+    f32x16 acc[DT];              // kKvBoth: dK1; kKvSplit: dV1 in the P waves, dK1 in the S waves
+    f32x16 acc2[TWO ? DT : 1];   // kKvBoth: dV1
 #pragma unroll
     for (int dt = 0; dt < DT; ++dt) acc[dt] = zero16();
 #pragma unroll
@@ -163,25 +150,8 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     const int wit_lo = jw / 32;
     const int wit_hi = ((jw + 31 + p.w1 - 1 < N - 1) ? jw + 31 + p.w1 - 1 : N - 1) / 32;
     const float c2 = p.scale_log2e;
-    // per-lane parts of the fragment addresses: plain row-major / transposed-read tiles, swizzled tiles
-    const int r_lane = c * PITCH + 16 * hf;
-    const int t_lane = tr_lane_off<D, L::TPITCH>(lane);
+    // per-lane parts of the fragment addresses of the swizzled tiles
     const SwzLane<D> swz_lane(lane);
-    auto row_frag = [&](const char *image, auto swz, int kk) {
-        if constexpr (decltype(swz)::value) return swz_lane.row_frag(image, kk);
-        else return ld_lds16(image + r_lane + 32 * kk);
-    };
-    auto tr_frag = [&](const char *image, auto swz, int k2s, int dt) {
-        if constexpr (decltype(swz)::value) {
-            return swz_lane.tr_frag(image, k2s, dt);
-        } else {
-            const u32x2 lo2 = lds_read_tr<D, L::TPITCH>(image + t_lane, 16 * k2s, 32 * dt);
-            const u32x2 hi2 = lds_read_tr<D, L::TPITCH>(image + t_lane, 16 * k2s + 8, 32 * dt);
-            return (u32x4){lo2[0], lo2[1], hi2[0], hi2[1]};
-        }
-    };
-    using ASwz = std::integral_constant<bool, L::A_SWZ>;
-    using BSwz = std::integral_constant<bool, L::B_SWZ>;
 
     // ---- pair iterator (g, it, blk, m): offsets 32 blk + 2m and 32 blk + 2m + 1 of query tile `it`, query head g
     // of the group.  (it, blk) is the staging unit: the q/do rows of the tile and the 63 k2/v2 rows that the 32
@@ -242,7 +212,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
             const int i = 32 * s.it + tid;
             const int icl = i < N ? i : N - 1;
             r_lse = p.lse[((int64_t)b * p.H + h) * N + icl] * kLog2e;
-            if constexpr (DK) r_del = p.delta[((int64_t)b * p.H + h) * N + icl];
+            r_del = p.delta[((int64_t)b * p.H + h) * N + icl];
         }
     };
     auto write_rows = [&]() {
@@ -254,7 +224,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
         }
         if (tid < 32) {
             reinterpret_cast<float *>(lds + L::LSES)[tid] = r_lse;
-            if constexpr (DK) reinterpret_cast<float *>(lds + L::LSES)[32 + tid] = r_del;
+            reinterpret_cast<float *>(lds + L::LSES)[32 + tid] = r_del;
         }
     };
 
@@ -262,25 +232,9 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     // thread, and a thread builds its piece of A and of B; 256 at D = 64, where threads 0-255
     // build A and threads 256-511 build B.  Either way a thread builds ITS piece for both steps
     // of the pair, so the q (dO) piece is read and unpacked once for two products.
-    // dv1 pass: the thread's q and dO pieces stay unpacked in registers for the whole query
-    // tile (the dk1 pass has no registers to spare and unpacks them once per pair)
     constexpr int PIECES = 32 * PPR;
     constexpr bool BOTH = PIECES == 512;
-    constexpr bool KEEP = MODE == kKvDv && BOTH;
     const int b_row = (tid % PIECES) / PPR, b_col = (tid % PPR) * 16;
-    float qx[8], ox[8];
-    auto unpack_own = [&]() {
-        const int row = b_row, col = b_col;
-        const u32x4 fq = ld_lds16(lds + L::QS + row * L::RP + col);
-        const u32x4 fo = ld_lds16(lds + L::DOS + row * L::RP + col);
-#pragma unroll
-        for (int w = 0; w < 4; ++w) {
-            qx[2 * w] = bf16_lo(fq[w]) * c2;
-            qx[2 * w + 1] = bf16_hi(fq[w]) * c2;
-            ox[2 * w] = bf16_lo(fo[w]);
-            ox[2 * w + 1] = bf16_hi(fo[w]);
-        }
-    };
     auto build = [&](const Pair &s, int buf) {
         const int row = b_row, col = b_col;
         const int dmax = dmax_of(s.it, s.blk);
@@ -298,33 +252,27 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                 r0[w] = pack_bf16(xv[2 * w] * bf16_lo(f0[w]), xv[2 * w + 1] * bf16_hi(f0[w]));
                 r1[w] = pack_bf16(xv[2 * w] * bf16_lo(f1[w]), xv[2 * w + 1] * bf16_hi(f1[w]));
             }
-            constexpr bool SWZ = IS_A ? L::A_SWZ : L::B_SWZ;
-            const int o = (IS_A ? L::AS : L::BS) + (SWZ ? swz_store_off<D>(row, col) : row * (IS_A ? L::A_PITCH : L::B_PITCH) + col);
+            const int o = (IS_A ? L::AS : L::BS) + swz_store_off<D>(row, col);
             *reinterpret_cast<u32x4 *>(stage + o) = r0;
             *reinterpret_cast<u32x4 *>(stage + L::STEP + o) = r1;
         };
-        if constexpr (KEEP) {
-            product(qx, L::K2S, std::true_type{});
-            product(ox, L::V2S, std::false_type{});
-        } else {
-            float xv[8];
-            auto unpack = [&](int xs, float f) {
-                const u32x4 fx = ld_lds16(lds + xs + row * L::RP + col);
+        float xv[8];
+        auto unpack = [&](int xs, float f) {
+            const u32x4 fx = ld_lds16(lds + xs + row * L::RP + col);
 #pragma unroll
-                for (int w = 0; w < 4; ++w) {
-                    xv[2 * w] = bf16_lo(fx[w]) * f;
-                    xv[2 * w + 1] = bf16_hi(fx[w]) * f;
-                }
-            };
-            if (BOTH || tid < PIECES) {
-                unpack(L::QS, c2);
-                product(xv, L::K2S, std::true_type{});
+            for (int w = 0; w < 4; ++w) {
+                xv[2 * w] = bf16_lo(fx[w]) * f;
+                xv[2 * w + 1] = bf16_hi(fx[w]) * f;
             }
-            if constexpr (BOTH) __builtin_amdgcn_sched_barrier(0);   // one product at a time: the dk1 pass has no registers for both
-            if (BOTH || (tid >= PIECES && tid < 2 * PIECES)) {
-                unpack(L::DOS, 1.f);
-                product(xv, L::V2S, std::false_type{});
-            }
+        };
+        if (BOTH || tid < PIECES) {
+            unpack(L::QS, c2);
+            product(xv, L::K2S, std::true_type{});
+        }
+        if constexpr (BOTH) __builtin_amdgcn_sched_barrier(0);   // one product at a time: no registers for both
+        if (BOTH || (tid >= PIECES && tid < 2 * PIECES)) {
+            unpack(L::DOS, 1.f);
+            product(xv, L::V2S, std::false_type{});
         }
         if (tid < 64) {
             const int e = tid >> 5, r = tid & 31;
@@ -334,7 +282,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
             char *st = stage + e * L::STEP;
             // (negated: the logit chains start from it)
             reinterpret_cast<float *>(st + L::LSE)[r] = valid ? -reinterpret_cast<const float *>(lds + L::LSES)[r] : -INFINITY;
-            if constexpr (DK) reinterpret_cast<float *>(st + L::DEL)[r] = valid ? -reinterpret_cast<const float *>(lds + L::LSES)[32 + r] : 0.f;
+            reinterpret_cast<float *>(st + L::DEL)[r] = valid ? -reinterpret_cast<const float *>(lds + L::LSES)[32 + r] : 0.f;
         }
     };
     // the -lse / -delta start values of the pair's chains (64 threads of the P group)
@@ -358,7 +306,6 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     write_rows();
     if (rw.g < p.G) issue_rows(rw);
     __syncthreads();
-    if constexpr (KEEP) unpack_own();
     build(nb, 0);
     next_pair(nb);
 
@@ -591,6 +538,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
         return;
     }
 
+    if constexpr (TWO) {
     for (int s = 0; s < npairs; ++s) {
         __syncthreads();
         if (s + 1 < npairs) {
@@ -601,7 +549,6 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                 next_unit(rw);
                 if (rw.g < p.G) issue_rows(rw);
                 __syncthreads();
-                if constexpr (KEEP) unpack_own();
             }
             build(nb, (s + 1) & 1);
             next_pair(nb);
@@ -611,7 +558,7 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
         next_pair(cur);
         if (!wave_active || it < wit_lo || it > wit_hi) continue;
 
-        // ---- S[i,j] (and dP[i,j]): rows = query rows of the tile, column = j
+        // ---- S[i,j] and dP[i,j]: rows = query rows of the tile, column = j
         // the chain starts from -lse_i log2(e) (stored negated by the build; -inf for dead rows), and A carries
         // scale * log2(e): the result is the exponent
         f32x16 X;
@@ -623,22 +570,20 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
             X[4 * a4 + 2] = l4.z;
             X[4 * a4 + 3] = l4.w;
         }
-        mfma_stream(NChain{}, [&](auto kk) { return row_frag(buf + L::AS, ASwz{}, kk); },
+        mfma_stream(NChain{}, [&](auto kk) { return swz_lane.row_frag(buf + L::AS, kk); },
                     [&](auto kk, const u32x4 &fr) { X = mfma32(fr, k1f[kk], X); });
+        // the accumulator starts at -delta_i (stored negated by the build): dP - delta costs no VALU work
         f32x16 dP;
-        if constexpr (DK) {
-            // the accumulator starts at -delta_i (stored negated by the build): dP - delta costs no VALU work
 #pragma unroll
-            for (int a4 = 0; a4 < 4; ++a4) {
-                const float4 d4 = *reinterpret_cast<const float4 *>(buf + L::DEL + (8 * a4 + 4 * hf) * 4);
-                dP[4 * a4] = d4.x;
-                dP[4 * a4 + 1] = d4.y;
-                dP[4 * a4 + 2] = d4.z;
-                dP[4 * a4 + 3] = d4.w;
-            }
-            mfma_stream(NChain{}, [&](auto kk) { return row_frag(buf + L::BS, BSwz{}, kk); },
-                        [&](auto kk, const u32x4 &fr) { dP = mfma32(fr, v1f[kk], dP); });
+        for (int a4 = 0; a4 < 4; ++a4) {
+            const float4 d4 = *reinterpret_cast<const float4 *>(buf + L::DEL + (8 * a4 + 4 * hf) * 4);
+            dP[4 * a4] = d4.x;
+            dP[4 * a4 + 1] = d4.y;
+            dP[4 * a4 + 2] = d4.z;
+            dP[4 * a4 + 3] = d4.w;
         }
+        mfma_stream(NChain{}, [&](auto kk) { return swz_lane.row_frag(buf + L::BS, kk); },
+                    [&](auto kk, const u32x4 &fr) { dP = mfma32(fr, v1f[kk], dP); });
         const bool full = (jw + 31 <= 32 * it) && (jw + p.w1 > 32 * it + 31);
         if (__builtin_expect(!full, 0)) {
             int base = 32 * it + 4 * hf - j;         // i - j for register 0
@@ -649,28 +594,19 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                 X[rr] = ok ? X[rr] : -INFINITY;
             }
         }
-        u32x4 pb[2];                 // dS with dk1, else P
-        u32x4 pv[TWO ? 2 : 1];       // P when both are produced
+        u32x4 pb[2];                 // dS
+        u32x4 pv[2];                 // P
 #pragma unroll
         for (int rr = 0; rr < 16; rr += 2) {
-            float p0 = fast_exp2(X[rr]);
-            float p1 = fast_exp2(X[rr + 1]);
-            if constexpr (TWO) pv[rr >> 3][(rr & 7) >> 1] = pack_bf16(p0, p1);
-            if constexpr (DK) {
-                p0 *= dP[rr];
-                p1 *= dP[rr + 1];
-            }
-            pb[rr >> 3][(rr & 7) >> 1] = pack_bf16(p0, p1);
+            const float p0 = fast_exp2(X[rr]);
+            const float p1 = fast_exp2(X[rr + 1]);
+            pv[rr >> 3][(rr & 7) >> 1] = pack_bf16(p0, p1);
+            pb[rr >> 3][(rr & 7) >> 1] = pack_bf16(p0 * dP[rr], p1 * dP[rr + 1]);
         }
-        if constexpr (DK)
-            mfma_stream(NProd{}, [&](auto x) { return tr_frag(buf + L::AS, ASwz{}, x / DT, x % DT); },
-                        [&](auto x, const u32x4 &fr) { acc[x % DT] = mfma32(fr, pb[x / DT], acc[x % DT]); });
-        else
-            mfma_stream(NProd{}, [&](auto x) { return tr_frag(buf + L::BS, BSwz{}, x / DT, x % DT); },
-                        [&](auto x, const u32x4 &fr) { acc[x % DT] = mfma32(fr, pb[x / DT], acc[x % DT]); });
-        if constexpr (TWO)
-            mfma_stream(NProd{}, [&](auto x) { return tr_frag(buf + L::BS, BSwz{}, x / DT, x % DT); },
-                        [&](auto x, const u32x4 &fr) { acc2[x % DT] = mfma32(fr, pv[x / DT], acc2[x % DT]); });
+        mfma_stream(NProd{}, [&](auto x) { return swz_lane.tr_frag(buf + L::AS, x / DT, x % DT); },
+                    [&](auto x, const u32x4 &fr) { acc[x % DT] = mfma32(fr, pb[x / DT], acc[x % DT]); });
+        mfma_stream(NProd{}, [&](auto x) { return swz_lane.tr_frag(buf + L::BS, x / DT, x % DT); },
+                    [&](auto x, const u32x4 &fr) { acc2[x % DT] = mfma32(fr, pv[x / DT], acc2[x % DT]); });
     }
 
     // ---- add the two groups of every slab and store
@@ -698,25 +634,22 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
     };
     if (pg == 1) {
         publish(acc, red);
-        if constexpr (TWO) publish(acc2, red + L::RED / 4);
+        publish(acc2, red + L::RED / 4);
     }
     __syncthreads();
     if (pg == 1 || !j_ok) return;
     collect(acc, red);
     char *dk1row = p.dk1.ptr + b * p.dk1.sb + (int64_t)j * p.dk1.sn + hk * p.dk1.sh + 16 * hf * 2;
     char *dv1row = p.dv1.ptr + b * p.dv1.sb + (int64_t)j * p.dv1.sn + hk * p.dv1.sh + 16 * hf * 2;
-    static_assert(!PARTS || TWO || SPLIT, "partial results exist for the kernels that form both outputs");
-    if constexpr (PARTS && TWO) {
-        store_row_f32<DT>(part_row(0), acc, kLn2);
+    if constexpr (PARTS) {
+        store_row_f32<DT>(part_row(0), acc, kLn2);   // A carried scale log2(e)
         collect(acc2, red + L::RED / 4);
         store_row_f32<DT>(part_row(1), acc2, 1.f);
-    } else if constexpr (!PARTS) {
-        if constexpr (DK) store_row<DT>(dk1row, acc, kLn2);   // A carried scale log2(e)
-        if constexpr (MODE == kKvDv) store_row<DT>(dv1row, acc, 1.f);
-        if constexpr (TWO) {
-            collect(acc2, red + L::RED / 4);
-            store_row<DT>(dv1row, acc2, 1.f);
-        }
+    } else {
+        store_row<DT>(dk1row, acc, kLn2);
+        collect(acc2, red + L::RED / 4);
+        store_row<DT>(dv1row, acc2, 1.f);
+    }
     }
 }
 

@@ -50,29 +50,30 @@ class _PartialsBudget:
     """Bytes of saved value partials alive per device (between a forward and the end of its
     backward).  The partials are ``w2`` times the size of ``q`` per call, so a deep model
     would otherwise keep ``layers * w2`` activations where the reference keeps ``layers``:
-    a call saves them only while (a) the call's buffer fits the per-call cap, (b) all live
-    buffers together stay below a fraction of the device's memory and (c) the buffer fits
-    half of what the device can still hand out.  Otherwise the backward recomputes, as the
-    reference does, at about 20 % more time per layer."""
+    a call saves them only while (a) the call's buffer fits the per-call cap and (b) all live
+    buffers together stay below a fraction of the device's total memory.  Otherwise the
+    backward recomputes, as the reference does, at about 20 % more time per layer.  The rule
+    looks at sizes only, never at how much memory happens to be free: the two backward paths
+    differ in the last bf16 digit of dV2, and a model's gradients must not depend on what
+    else the allocator holds."""
 
     def __init__(self):
         self.live = {}
+        self.total = {}
         self.lock = threading.Lock()
 
-    def admit(self, nbytes: int, device, mem_info=None) -> bool:
+    def admit(self, nbytes: int, device, total_memory=None) -> bool:
         if nbytes <= 0 or nbytes > save_partials_max_bytes():
             return False
         index = torch.device(device).index
         index = torch.cuda.current_device() if index is None else index
-        if mem_info is None:
-            free, total = torch.cuda.mem_get_info(index)
-            # blocks the caching allocator holds but has not handed out are available too
-            free += torch.cuda.memory_reserved(index) - torch.cuda.memory_allocated(index)
-        else:
-            free, total = mem_info
         with self.lock:
+            if total_memory is None:
+                if index not in self.total:
+                    self.total[index] = torch.cuda.get_device_properties(index).total_memory
+                total_memory = self.total[index]
             live = self.live.get(index, 0)
-            if live + nbytes > save_partials_total_fraction() * total or nbytes > free // 2:
+            if live + nbytes > save_partials_total_fraction() * total_memory:
                 return False
             self.live[index] = live + nbytes
         return True
@@ -145,8 +146,14 @@ class SlidingTwoSimplicialAttention(Function):
         t_save = m_save = None
         t_bytes = lib.sa2_saved_t_bytes(prob) + lib.sa2_saved_m_bytes(prob)
         if needs_grad and partials_budget.admit(t_bytes, q.device):
-            t_save = torch.empty(lib.sa2_saved_t_bytes(prob), dtype=torch.uint8, device=q.device)
-            m_save = torch.empty((batch, heads, w2, seq_len), dtype=torch.float32, device=q.device)
+            try:
+                t_save = torch.empty(lib.sa2_saved_t_bytes(prob), dtype=torch.uint8, device=q.device)
+                m_save = torch.empty((batch, heads, w2, seq_len), dtype=torch.float32, device=q.device)
+            except BaseException:
+                # (no buffer to hang the release on: give the admitted bytes back here)
+                index = q.device.index if q.device.index is not None else torch.cuda.current_device()
+                partials_budget.release(t_bytes, index)
+                raise
             partials_budget.track(t_save, t_bytes)
         with torch.cuda.device_of(q):
             _native.check(lib.sa2_fwd(prob, *(_native.tensor_arg(t) for t in (q, k1, k2, v1, v2, out)),

@@ -140,3 +140,49 @@ def test_config1_full_causal_against_dense_naive_attend():
     assert out.dtype is torch.float32 and out.shape == (b, n, h, d)
     grads = torch.autograd.grad(out, ts, to_kernel(dout).cuda())
     U.check_all(out, grads, to_kernel(ref_out.detach()), [to_kernel(t) for t in ref_grads], unit_variance=True)
+
+
+@pytest.mark.parametrize('n, seed', [(8192, 12), (32768, 13)])
+def test_full_length_slices_with_unit_variance_inputs(n, seed):
+    """One (batch, head) slice at the sequence lengths of configs 3 and 4 (D = 128, w1 = 512, w2 = 32) with
+    UNSCALED N(0,1) inputs: the benchmark distribution N(0,1)/sqrt(D) makes outputs of order 1e-4, where only
+    the relative bound binds; here logits have unit variance and outputs are of order one, so the elementwise
+    criterion binds on every row of the full sequence.  Against the banded fp32 oracle, with the reference's own
+    tolerances for such inputs (tests/test_triton.py:104-115) plus the relative Frobenius bound."""
+    d, w1, w2 = 128, 512, 32
+    ins = U.make_inputs(1, n, 1, 1, d, seed=seed, std=1.0)
+    ref_out, _, ref_grads = U.oracle_fwd_bwd(*ins, w1, w2)
+    out, grads = _run(*(t.cuda() for t in ins), w1, w2)
+    U.check_all(out.cpu(), [t.cpu() for t in grads], ref_out, ref_grads, unit_variance=True)
+
+
+def test_config5_full_training_step_is_finite_and_deterministic():
+    """benchmark config 5 at full size: the byte-level language model (depth 12, dim 512, 8 heads of 64 on 4
+    key/value heads, every 2nd layer simplicial with w1 = 512, w2 = 32) on a batch of 8 x 2048 random bytes, bf16.
+    One forward + backward: the loss of the untrained model is close to ln 256, every gradient is finite, and a
+    second run gives the same loss and the same gradients bit for bit (no atomics anywhere on the path)."""
+    import math
+    from simplicial_attention_amd.two_simplicial_transformer import TwoSimplicialLM
+    torch.manual_seed(4)
+    lm = TwoSimplicialLM(num_tokens=256, dim=512, depth=12, max_seq_len=2048, dim_head=64, heads=8,
+                         two_simplicial_attn_every=2, transformer_kwargs=dict(key_value_heads=4)).bfloat16().cuda()
+    tokens = torch.randint(0, 256, (8, 2049), generator=torch.Generator().manual_seed(6)).cuda()
+
+    def run():
+        lm.zero_grad(set_to_none=True)
+        loss = lm(tokens, return_loss=True)
+        loss.backward()
+        torch.cuda.synchronize()
+        return loss.item(), {k: p.grad.clone() for k, p in lm.named_parameters()}
+    loss_a, grads_a = run()
+    loss_b, grads_b = run()
+    print('   loss', loss_a, 'ln 256 =', math.log(256), flush=True)
+    assert math.isfinite(loss_a) and abs(loss_a - math.log(256)) <= 0.5, loss_a
+    assert loss_a == loss_b
+    for name, g in grads_a.items():
+        assert torch.isfinite(g).all(), name
+        assert float(g.float().norm()) > 0, name
+    # the simplicial layers' own parameters must be reproduced bit for bit (the library has no atomics); the other
+    # layers go through torch's kernels, which are deterministic for these shapes too
+    for name, g in grads_a.items():
+        assert torch.equal(g, grads_b[name]), name
