@@ -195,6 +195,46 @@ def traffic_from(directory):
     json.dump(rec, open(TRAFFIC_FILE, 'w'), indent=1, sort_keys=True)
     print(json.dumps(rec))
 
+def mfma_mix_rates(iters=2048, workgroups=1024):
+    """What the chip sustains on an instruction mix (profiling build of the library, sa2_prof_mix.hpp): a loop of
+    independent bf16 MFMAs, two waves per SIMD, with 0 / 4+1+1 / 7+1+2 (VALU + exponential + 1 KiB LDS read) other
+    instructions per MFMA, on random and on constant operands.  The nominal peak assumes the nominal clock, which the
+    chip holds only on operands that do not toggle."""
+    import ctypes
+    import torch
+    from simplicial_attention_amd import _native
+    plib = _native.load_profiling()
+    fn = plib.sa2_prof_mfma_mix
+    fn.restype = ctypes.c_int
+    fn.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    dev = torch.device('cuda:0')
+    out = torch.empty(workgroups * 512, dtype=torch.float32, device=dev)
+    clocks = torch.zeros(2, dtype=torch.int64, device=dev)
+    stream = torch.cuda.current_stream()
+    g = torch.Generator(device='cpu').manual_seed(7)
+    data = {'random': torch.randn(32768, generator=g).bfloat16().to(dev), 'constant': torch.ones(32768).bfloat16().to(dev)}
+    mixes = {0: 'mfma_only', 1: 'plus_4_valu_1_exp_1_lds_read_per_mfma', 2: 'plus_7_valu_1_exp_2_lds_reads_per_mfma'}
+    res = {}
+    for dname, ops in data.items():
+        for mix, mname in mixes.items():
+            best = None
+            for _ in range(3):
+                a, b_ = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                a.record(stream)
+                rc = fn(ops.data_ptr(), out.data_ptr(), clocks.data_ptr(), mix, workgroups, iters, stream.cuda_stream)
+                b_.record(stream)
+                torch.cuda.synchronize()
+                if rc != 0:
+                    raise RuntimeError(plib.sa2_last_error().decode())
+                ms = a.elapsed_time(b_)
+                best = ms if best is None or ms < best else best
+            c = clocks.cpu()
+            tf = workgroups * 8 * iters * 16 * 32768 / (best * 1e-3) / 1e12
+            res['%s_operands__%s' % (dname, mname)] = {'tflops': round(tf, 1), 'frac_of_nominal_peak': round(tf / PEAK_BF16_TFLOPS, 4),
+                                                        'shader_clock_mhz': round(100.0 * int(c[0]) / max(int(c[1]), 1), 0)}
+    return res
+
+
 def time_raw_workload(name, steps=5, warmup=2):
     """forward + backward of the raw kernel path at workload `name` through the autograd Function: ms per step,
     TFLOP/s on the 18*D*B*H*P count and the fraction of the bf16 MFMA peak."""
@@ -327,7 +367,7 @@ def main():
     ap.add_argument('--no-other-workloads', dest='other_workloads', action='store_false',
                     help='skip the other benchmark workloads (config 4, the config-5 layer and training step, the config-2 module) that the default run times after config 3')
     ap.add_argument('--traffic-from', default=None, metavar='DIR', help='no GPU work: read the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE passes under DIR and write profiles/hbm_traffic.json')
-    ap.add_argument('--only', default=None, help='time only this entry through the C ABI (fwd, bwd_delta, bwd_dq_dkv2, bwd_dkv1, bwd_dq_dk2_pass), `copy`: a 1 GiB device copy that calibrates HBM counters; `module_cfg2`: the module forward of config 2 and the fused qkv-norm kernel; `train_cfg5`: one training step of the config-5 language model; for profiling')
+    ap.add_argument('--only', default=None, help='time only this entry through the C ABI (fwd, bwd_delta, bwd_dq_dkv2, bwd_dkv1, bwd_dq_dk2_pass), `mfma_mix`: the MFMA rates this chip sustains on three instruction mixes with random and constant operands; `copy`: a 1 GiB device copy that calibrates HBM counters; `module_cfg2`: the module forward of config 2 and the fused qkv-norm kernel; `train_cfg5`: one training step of the config-5 language model; for profiling')
     args = ap.parse_args()
     if args.traffic_from:
         traffic_from(args.traffic_from)
@@ -353,6 +393,9 @@ def main():
         return
     if args.only == 'module_cfg2':
         print(json.dumps(time_module_cfg2()))
+        return
+    if args.only == 'mfma_mix':
+        print(json.dumps(mfma_mix_rates()))
         return
     if args.only == 'copy':
         # plain device copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters
@@ -522,6 +565,13 @@ def main():
         'kernels': kernels,
         'roofline': roofline,
     }
+    # what the MFMA pipe sustains on this chip, measured in the same run: the nominal peak holds for operands that do
+    # not toggle; on random operands the clock drops under the power limit
+    sustained = mfma_mix_rates(iters=1024)
+    roofline['sustained_on_this_chip'] = sustained
+    rnd = sustained['random_operands__mfma_only']['tflops']
+    roofline['frac_of_sustained_random_operand_mfma_rate'] = round(achieved / rnd, 4)
+    result['frac_of_sustained_random_operand_mfma_rate'] = round(value / rnd, 4)
     if args.other_workloads and args.workload == 'cfg3_raw_kernel_b4_h8_n8192_d128_w512_w32':
         # the other benchmark workloads, timed in the same run (each at least 5 steps)
         torch.cuda.empty_cache()

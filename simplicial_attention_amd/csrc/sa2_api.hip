@@ -17,6 +17,9 @@
 #include "sa2_lds.hpp"
 #include "sa2_qkv_norm.hpp"
 #include "sa2_fwd.hpp"
+#ifdef SA2_PROFILING
+#include "sa2_prof_mix.hpp"
+#endif
 
 namespace {
 
@@ -556,5 +559,23 @@ int sa2_qkv_norm_bwd(const sa2_problem *prob, const void *qkv, int64_t row_strid
     hipLaunchKernelGGL(sa2::qkv_norm_dw_kernel, dim3((n + 15) / 16), dim3(256), 0, s, np.dw_part, dw, blocks, n);
     return after_launch("qkv norm weight gradients");
 }
+
+#ifdef SA2_PROFILING
+// Profiling build only: the instruction-mix loop of sa2_prof_mix.hpp.  `operands`: 64 KiB of bf16 values on the device,
+// `out`: workgroups * 512 floats, `clocks`: two 64-bit counters (shader clock, 100 MHz clock) of workgroup 0.  Each SIMD
+// executes workgroups / 256 * iters * 32 MFMAs (two waves of 16).  mix: 0 = MFMAs only; 1 = + 4 VALU, 1 exponential and
+// 1 LDS fragment read per MFMA; 2 = + 7 VALU, 1 exponential and 2 LDS fragment reads per MFMA.
+int sa2_prof_mfma_mix(const void *operands, float *out, unsigned long long *clocks, int mix, int workgroups, int iters, void *hip_stream) {
+    if (!operands || !out || !clocks) return fail(SA2_ERR_NULL_POINTER, "operands, out or clocks is NULL");
+    if (workgroups < 1 || iters < 1) return fail(SA2_ERR_BAD_SHAPE, "workgroups and iters must be positive");
+    hipStream_t s = static_cast<hipStream_t>(hip_stream);
+    const char *src = static_cast<const char *>(operands);
+    if (mix == 0) hipLaunchKernelGGL((sa2::prof_mix_kernel<0, 0, 0>), dim3(workgroups), dim3(512), 0, s, src, out, iters, clocks);
+    else if (mix == 1) hipLaunchKernelGGL((sa2::prof_mix_kernel<4, 1, 1>), dim3(workgroups), dim3(512), 0, s, src, out, iters, clocks);
+    else if (mix == 2) hipLaunchKernelGGL((sa2::prof_mix_kernel<7, 1, 2>), dim3(workgroups), dim3(512), 0, s, src, out, iters, clocks);
+    else return fail(SA2_ERR_UNSUPPORTED, "mix %d is not one of 0, 1, 2", mix);
+    return after_launch("instruction-mix loop");
+}
+#endif
 
 }  // extern "C"
