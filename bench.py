@@ -36,6 +36,7 @@ WORKLOADS = {
     'cfg4_long_context_b1_h16_n32768_d128_w512_w32': (1, 16, 16, 32768, 128, 512, 32),
     'cfg5_layer_b8_h8_kv4_n2048_d64_w512_w32': (8, 8, 4, 2048, 64, 512, 32),
     'tiny_b1_h2_n512_d128_w512_w32': (1, 2, 2, 512, 128, 512, 32),
+    'wide_heads_b2_h8_n4096_d256_w512_w32': (2, 8, 8, 4096, 256, 512, 32),
 }
 
 
@@ -125,6 +126,8 @@ ENTRY_KERNEL = {'fwd': 'fwd', 'bwd_dq_dk2_pass': 'bwd_q_kernel', 'bwd_dkv1': 'bw
 
 
 def kernel_symbol(entry, D, w2):
+    if D == 256:
+        return {'fwd': 'sa2::fwd_wide_kernel<256>', 'bwd_dq_dk2_pass': 'sa2::bwd_wide_q_kernel<256>', 'bwd_dkv1': 'sa2::bwd_wide_kv_kernel<256>'}.get(entry)
     if entry == 'fwd':
         return 'sa2::fwd_kernel<%d>' % D
     if entry == 'bwd_dq_dk2_pass':
@@ -463,7 +466,7 @@ def main():
     # the forward's per-offset value partials, as the autograd Function keeps them
     saved = t_save = m_save = None
     from simplicial_attention_amd.two_simplicial_attention import save_partials_max_bytes
-    if lib.sa2_saved_t_bytes(prob) <= save_partials_max_bytes():
+    if 0 < lib.sa2_saved_t_bytes(prob) <= save_partials_max_bytes():      # (0: this head dimension keeps no partials)
         t_save = torch.empty(lib.sa2_saved_t_bytes(prob), dtype=torch.uint8, device=dev)
         m_save = torch.empty(lib.sa2_saved_m_bytes(prob), dtype=torch.uint8, device=dev)
         saved = _native.saved_arg(t_save, m_save)

@@ -17,6 +17,7 @@
 #include "sa2_lds.hpp"
 #include "sa2_qkv_norm.hpp"
 #include "sa2_fwd.hpp"
+#include "sa2_wide.hpp"
 #ifdef SA2_PROFILING
 #include "sa2_prof_mix.hpp"
 #endif
@@ -43,8 +44,8 @@ int check_problem(const sa2_problem *p) {
     if (p->w1 < 1 || p->w2 < 1) return fail(SA2_ERR_BAD_SHAPE, "windows w1=%d w2=%d must be >= 1", p->w1, p->w2);
     if (p->causal != 1) return fail(SA2_ERR_UNSUPPORTED, "only causal=1 is defined for the sliding windows");
     if (p->dtype != SA2_BF16) return fail(SA2_ERR_UNSUPPORTED, "dtype %d is not supported (bf16 only)", p->dtype);
-    if (p->dim_head != 32 && p->dim_head != 64 && p->dim_head != 128)
-        return fail(SA2_ERR_UNSUPPORTED, "dim_head=%d is not supported (32, 64 or 128)", p->dim_head);
+    if (p->dim_head != 32 && p->dim_head != 64 && p->dim_head != 128 && p->dim_head != 256)
+        return fail(SA2_ERR_UNSUPPORTED, "dim_head=%d is not supported (32, 64, 128 or 256)", p->dim_head);
     if (!(p->scale > 0.f) || !std::isfinite(p->scale)) return fail(SA2_ERR_BAD_SHAPE, "scale must be positive and finite");
     if ((int64_t)p->batch * p->heads * ((p->seq_len + 31) / 32) > 0x7fffffffll)
         return fail(SA2_ERR_BAD_SHAPE, "problem too large for a 1-D grid");
@@ -95,19 +96,34 @@ int after_launch(const char *what) {
         if (rc_ != SA2_OK) return rc_; \
     } while (0)
 
-// Runs `stmt` with the compile-time constant DH set to the problem's head dimension (validated by check_problem).
-#define SA2_FOR_DIM_HEAD(dim_head, stmt)        \
+// Head dimension 256 runs kernels of its own (sa2_wide.hpp), which keep no forward partials.
+constexpr int kWideDimHead = 256;
+
+// Runs the statement with the compile-time constant DH set to the problem's head dimension (validated by
+// check_problem): the kernels built for head dimensions 32, 64 and 128 ...
+#define SA2_FOR_DIM_HEAD(dim_head, ...)         \
     do {                                        \
         if ((dim_head) == 128) {                \
             constexpr int DH = 128;             \
-            stmt;                               \
+            __VA_ARGS__;                        \
         } else if ((dim_head) == 64) {          \
             constexpr int DH = 64;              \
-            stmt;                               \
+            __VA_ARGS__;                        \
         } else {                                \
             constexpr int DH = 32;              \
-            stmt;                               \
+            __VA_ARGS__;                        \
         }                                       \
+    } while (0)
+
+// ... and the kernels that every head dimension shares
+#define SA2_FOR_ANY_DIM_HEAD(dim_head, ...)             \
+    do {                                                \
+        if ((dim_head) == kWideDimHead) {               \
+            constexpr int DH = kWideDimHead;            \
+            __VA_ARGS__;                                \
+        } else {                                        \
+            SA2_FOR_DIM_HEAD(dim_head, __VA_ARGS__);    \
+        }                                               \
     } while (0)
 
 // Scratch of sa2_bwd_noalloc: delta rows followed by the dK2/dV2 partial rows.  A file-scope device
@@ -147,10 +163,11 @@ int sa2_version(void) { return SA2_VERSION; }
 const char *sa2_last_error(void) { return g_err; }
 
 int sa2_supported(int32_t dim_head, int32_t w1, int32_t w2, int32_t dtype) {
-    return (dim_head == 32 || dim_head == 64 || dim_head == 128) && w1 >= 1 && w2 >= 1 && dtype == SA2_BF16;
+    return (dim_head == 32 || dim_head == 64 || dim_head == 128 || dim_head == kWideDimHead) && w1 >= 1 && w2 >= 1 && dtype == SA2_BF16;
 }
 
-static int check_saved(const sa2_saved *saved) {
+static int check_saved(const sa2_problem *prob, const sa2_saved *saved) {
+    if (prob->dim_head == kWideDimHead) return fail(SA2_ERR_UNSUPPORTED, "dim_head=%d keeps no forward partials: pass saved = NULL", prob->dim_head);
     if (!saved->t || !saved->m) return fail(SA2_ERR_NULL_POINTER, "saved->t or saved->m is NULL");
     if ((reinterpret_cast<uintptr_t>(saved->t) & 15) != 0) return fail(SA2_ERR_ALIGNMENT, "saved->t must be 16-byte aligned");
     return SA2_OK;
@@ -158,11 +175,13 @@ static int check_saved(const sa2_saved *saved) {
 
 int64_t sa2_saved_t_bytes(const sa2_problem *prob) {
     if (check_problem(prob) != SA2_OK) return -1;
+    if (prob->dim_head == kWideDimHead) return 0;
     return (int64_t)prob->batch * prob->heads * prob->w2 * ((prob->seq_len + 31) / 32) * 32 * prob->dim_head * 2;
 }
 
 int64_t sa2_saved_m_bytes(const sa2_problem *prob) {
     if (check_problem(prob) != SA2_OK) return -1;
+    if (prob->dim_head == kWideDimHead) return 0;
     return (int64_t)prob->batch * prob->heads * prob->w2 * prob->seq_len * 4;
 }
 
@@ -189,12 +208,15 @@ int sa2_fwd(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, 
     k.lse = lse;
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
     if (saved) {
-        SA2_TRY(check_saved(saved));
+        SA2_TRY(check_saved(prob, saved));
         k.t_save = static_cast<char *>(saved->t);
         k.m_save = saved->m;
     }
     const int grid = prob->batch * prob->heads * ((prob->seq_len + 31) / 32);
-    SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL(sa2::fwd_kernel<DH>, dim3(grid), dim3(512), 0, s, k));
+    if (prob->dim_head == kWideDimHead)
+        hipLaunchKernelGGL(sa2::fwd_wide_kernel<kWideDimHead>, dim3(grid), dim3(256), 0, s, k);
+    else
+        SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL(sa2::fwd_kernel<DH>, dim3(grid), dim3(512), 0, s, k));
     return after_launch("forward");
 }
 
@@ -215,7 +237,7 @@ int sa2_bwd_delta(const sa2_problem *prob, const sa2_tensor *out, const sa2_tens
     int lanes_per_row = prob->dim_head / 8;
     int rows_per_block = 256 / lanes_per_row;
     int grid = (int)((rows + rows_per_block - 1) / rows_per_block);
-    SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL(sa2::delta_kernel<DH>, dim3(grid), dim3(256), 0, s, k));
+    SA2_FOR_ANY_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL(sa2::delta_kernel<DH>, dim3(grid), dim3(256), 0, s, k));
     return after_launch("delta");
 }
 
@@ -273,6 +295,7 @@ static constexpr int kComputeUnits = 256;
 static int cu_count() { return kComputeUnits; }
 
 static bool dkv1_in_parts(const sa2_problem *prob) {
+    if (prob->dim_head == kWideDimHead) return false;
     const int ntile = (prob->seq_len + 127) / 128;
     const int64_t grid = (int64_t)prob->batch * prob->kv_heads * ntile;
     const int64_t ragged = (prob->w1 + 127) / 128 + 1;          // slabs per sequence with a shortened range of query tiles
@@ -334,7 +357,7 @@ static int prepare_dq_dkv2(const sa2_problem *prob, const sa2_tensor *q, const s
     // replaced by a kernel that streams T once
     out->use_saved = saved_given;
     if (saved) {
-        SA2_TRY(check_saved(saved));
+        SA2_TRY(check_saved(prob, saved));
         k.t_save = static_cast<char *>(saved->t);
         k.m_save = saved->m;
     }
@@ -342,6 +365,11 @@ static int prepare_dq_dkv2(const sa2_problem *prob, const sa2_tensor *q, const s
 }
 
 static int launch_q_mfma(const sa2_problem *prob, const QLaunch &L, int pass, hipStream_t s) {
+    if (prob->dim_head == kWideDimHead) {
+        // one kernel forms dQ and both sets of partial rows
+        hipLaunchKernelGGL(sa2::bwd_wide_q_kernel<kWideDimHead>, dim3(L.grid), dim3(256), 0, s, L.k, L.ws, L.halo);
+        return after_launch("dq/dk2/dv2");
+    }
     SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL((sa2::bwd_q_kernel<DH, true>), dim3(L.grid), dim3(512), 0, s, L.k, L.ws, L.halo));
     if (pass != 1 && !L.use_saved)
         SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL((sa2::bwd_q_kernel<DH, false>), dim3(L.grid), dim3(512), 0, s, L.k, L.ws, L.halo));
@@ -359,7 +387,7 @@ static int launch_q_combine(const sa2_problem *prob, const QLaunch &L, hipStream
     const int rows_per_block = 256 / (prob->dim_head / 8);
     const int cgrid = (int)((rows + rows_per_block - 1) / rows_per_block);
     const int with_dv2 = L.use_saved ? 0 : 1;
-    SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL(sa2::dk2_dv2_combine_kernel<DH>, dim3(cgrid), dim3(256), 0, s, L.k, L.ws, 32 + L.halo, with_dv2));
+    SA2_FOR_ANY_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL(sa2::dk2_dv2_combine_kernel<DH>, dim3(cgrid), dim3(256), 0, s, L.k, L.ws, 32 + L.halo, with_dv2));
     return after_launch("dk2/dv2 combine");
 }
 
@@ -388,6 +416,11 @@ static int launch_dkv1(const sa2_problem *prob, const sa2_tensor *q, const sa2_t
     k.dv1 = dev(dv1);
     k.kv_parts = parts;
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
+    if (prob->dim_head == kWideDimHead) {
+        const int wgrid = prob->batch * prob->kv_heads * ((prob->seq_len + 31) / 32);
+        hipLaunchKernelGGL(sa2::bwd_wide_kv_kernel<kWideDimHead>, dim3(wgrid), dim3(256), 0, s, k);
+        return after_launch("dk1/dv1");
+    }
     const int grid = prob->batch * prob->kv_heads * ((prob->seq_len + 127) / 128);
     // dim_head 128: the two waves of a slab split the contractions; dim_head 64 and 32: each wave forms both outputs
     if (parts) {
@@ -523,7 +556,7 @@ int sa2_qkv_norm_fwd(const sa2_problem *prob, const void *qkv, int64_t row_strid
     np.eps = eps;
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
     const int grid = norm_groups(prob);
-    SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL(sa2::qkv_norm_fwd_kernel<DH>, dim3(grid), dim3(256), 0, s, np));
+    SA2_FOR_ANY_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL(sa2::qkv_norm_fwd_kernel<DH>, dim3(grid), dim3(256), 0, s, np));
     return after_launch("qkv norm forward");
 }
 
@@ -553,7 +586,7 @@ int sa2_qkv_norm_bwd(const sa2_problem *prob, const void *qkv, int64_t row_strid
     hipStream_t s = static_cast<hipStream_t>(hip_stream);
     const int groups = norm_groups(prob);
     const int blocks = groups < kNormMaxBlocks ? groups : kNormMaxBlocks;
-    SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL(sa2::qkv_norm_bwd_kernel<DH>, dim3(blocks), dim3(256), 0, s, np, groups));
+    SA2_FOR_ANY_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL(sa2::qkv_norm_bwd_kernel<DH>, dim3(blocks), dim3(256), 0, s, np, groups));
     SA2_TRY(after_launch("qkv norm backward"));
     const int n = 5 * prob->dim_head;
     hipLaunchKernelGGL(sa2::qkv_norm_dw_kernel, dim3((n + 15) / 16), dim3(256), 0, s, np.dw_part, dw, blocks, n);

@@ -78,7 +78,7 @@ class HigherOrderAttention(nn.Module):
     def _can_fuse(self, qkv):
         dh = self.split_dims[0] // self.heads
         return (self.fused_qkv_norm and self.qk_rmsnorm and self.kv_sets == 2 and not self.head_first_dim
-                and qkv.is_cuda and qkv.dtype is torch.bfloat16 and dh in (32, 64, 128)
+                and qkv.is_cuda and qkv.dtype is torch.bfloat16 and dh in (32, 64, 128, 256)
                 and self.split_dims[1] == self.split_dims[2]
                 and all(n.eps == self.q_norm.eps for n in (*self.k_norms, *self.v_norms)))
 

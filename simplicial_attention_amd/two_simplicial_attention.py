@@ -131,7 +131,7 @@ class SlidingTwoSimplicialAttention(Function):
             raise ValueError('window sizes must be at least 1')
         lib = _native.load()
         if not lib.sa2_supported(dim, w1, w2, _native.SA2_BF16):
-            raise NotImplementedError(f'dim_head={dim}, w1={w1}, w2={w2} is not covered by the kernels (dim_head 32, 64 or 128)')
+            raise NotImplementedError(f'dim_head={dim}, w1={w1}, w2={w2} is not covered by the kernels (dim_head 32, 64, 128 or 256)')
 
         q, k1, k2, v1, v2 = (_unit_inner_stride(t) for t in tensors)
         scale = dim ** -0.5 if scale is None else float(scale)
@@ -145,7 +145,8 @@ class SlidingTwoSimplicialAttention(Function):
         # they fit the budget: dV2 then needs no recomputation of the attention weights
         t_save = m_save = None
         t_bytes = lib.sa2_saved_t_bytes(prob) + lib.sa2_saved_m_bytes(prob)
-        if needs_grad and partials_budget.admit(t_bytes, q.device):
+        # (a size of 0: this head dimension's kernels keep no partials)
+        if needs_grad and t_bytes > 0 and partials_budget.admit(t_bytes, q.device):
             try:
                 t_save = torch.empty(lib.sa2_saved_t_bytes(prob), dtype=torch.uint8, device=q.device)
                 m_save = torch.empty((batch, heads, w2, seq_len), dtype=torch.float32, device=q.device)
@@ -214,8 +215,8 @@ def sliding_two_simplicial_attn(
 
     Beyond the reference (whose kernels are written for bf16 and a head dimension of
     64): float16 and float32 tensors are computed in bfloat16 and the result returned
-    in the input dtype; any head dimension up to 128, and a value head dimension
-    different from the query/key one, are zero-padded to the kernels' 32, 64 or 128
+    in the input dtype; any head dimension up to 256, and a value head dimension
+    different from the query/key one, are zero-padded to the kernels' 32, 64, 128 or 256
     (padded query/key channels add nothing to the logits, padded value channels give
     zero outputs that are sliced off; the softmax scale stays that of the true
     query/key dimension).
@@ -231,11 +232,11 @@ def sliding_two_simplicial_attn(
     if k1.shape[-1] != dim_qk or k2.shape[-1] != dim_qk or v2.shape[-1] != dim_v:
         raise ValueError('q, k1, k2 must share one head dimension and v1, v2 another')
     dim = max(dim_qk, dim_v)
-    if dim > 128:
-        raise NotImplementedError(f'head dimension {dim} is not covered by the kernels (at most 128)')
-    if dtype is torch.bfloat16 and dim_qk == dim_v and dim in (32, 64, 128):
+    if dim > 256:
+        raise NotImplementedError(f'head dimension {dim} is not covered by the kernels (at most 256)')
+    if dtype is torch.bfloat16 and dim_qk == dim_v and dim in (32, 64, 128, 256):
         return _sliding_two_simplicial_attn(q, k1, k2, v1, v2, w1, w2, causal)
-    dim_kernel = 32 if dim <= 32 else (64 if dim <= 64 else 128)
+    dim_kernel = next(d for d in (32, 64, 128, 256) if dim <= d)
 
     def prepare(t):
         t = t.to(torch.bfloat16)

@@ -43,13 +43,26 @@ def test_supported_matrix(lib):
     assert lib.sa2_supported(64, 8192, 8192, 0) == 1
     assert lib.sa2_supported(32, 512, 32, 0) == 1
     assert lib.sa2_supported(96, 512, 32, 0) == 0
-    assert lib.sa2_supported(256, 512, 32, 0) == 0
+    assert lib.sa2_supported(256, 512, 32, 0) == 1
+    assert lib.sa2_supported(512, 512, 32, 0) == 0
     assert lib.sa2_supported(128, 0, 32, 0) == 0
     assert lib.sa2_supported(128, 512, 32, 1) == 0
 
 
 def _dummy(ptr=0x1000, sb=1024, sn=128, sh=8):
     return _native.TensorArg(ptr, sb, sn, sh)
+
+
+def test_head_dimension_256_keeps_no_forward_partials(lib):
+    """The kernels of head dimension 256 recompute in the backward: the size queries say 0 and a call that passes
+    saved partials anyway is refused before any launch."""
+    prob = _native.problem(1, 64, 2, 1, 256, 512, 32, True, 256 ** -0.5)
+    assert lib.sa2_saved_t_bytes(prob) == 0 and lib.sa2_saved_m_bytes(prob) == 0
+    assert lib.sa2_bwd_workspace_bytes(prob) == 2 * 1 * 2 * 2 * (32 + 31) * 256 * 4
+    t = _dummy()
+    saved = _native.Saved(0x4000, 0x8000)
+    assert lib.sa2_fwd(prob, t, t, t, t, t, t, None, ctypes.c_void_p(0x2000), ctypes.byref(saved), None) == 3
+    assert b'256' in lib.sa2_last_error()
 
 
 def test_argument_validation_happens_before_any_launch(lib):
@@ -123,7 +136,7 @@ def test_function_rejects_what_the_kernels_do_not_cover():
 
 def test_wrapper_checks_head_dimensions_and_dtypes():
     q = torch.randn(1, 16, 2, 64)
-    wide = torch.randn(1, 16, 2, 160)
+    wide = torch.randn(1, 16, 2, 264)
     with pytest.raises(NotImplementedError):     # beyond the kernels' largest head dimension
         S.sliding_two_simplicial_attn(wide, (wide, wide), (wide, wide))
     with pytest.raises(ValueError):              # k2 with a head dimension of its own

@@ -32,6 +32,10 @@ CASES = [
     (2, 333, 4, 2, 32, 100, 32),      # head dimension 32, ragged N, grouped heads
     (1, 200, 2, 1, 32, 48, 70),       # head dimension 32, several offset blocks
     (1, 19, 2, 2, 32, 512, 32),       # head dimension 32, less than one tile
+    (1, 128, 2, 2, 256, 64, 32),      # head dimension 256 (kernels of their own: the waves of a workgroup split the head dimension)
+    (2, 300, 4, 2, 256, 100, 40),     # head dimension 256, ragged N, grouped heads, second window beyond 32
+    (1, 45, 2, 1, 256, 512, 32),      # head dimension 256, windows wider than the sequence
+    (1, 1, 1, 1, 256, 512, 32),       # head dimension 256, a single row
 ]
 
 
@@ -71,7 +75,8 @@ def test_seeded_random_shapes(b, n, hq, hk, d, w1, w2):
     U.check_all(out, grads, ref_out, ref_grads)
 
 
-def test_large_and_drifting_logits():
+@pytest.mark.parametrize('d', [128, 256])
+def test_large_and_drifting_logits(d):
     """Logits that grow along the sequence by far more than 2^64 per window: exercises
     the paths of the forward that move the softmax reference point while accumulators
     hold data.  q and k2 hold powers of two and the softmax scale is chosen so that
@@ -81,7 +86,7 @@ def test_large_and_drifting_logits():
     they round q * k1 * scale to bf16, triton_two_simplicial_attention.py:150-152, 182)."""
     import math
     from simplicial_attention_amd import SlidingTwoSimplicialAttention
-    b, n, h, d, w1, w2 = 1, 256, 2, 128, 96, 16
+    b, n, h, w1, w2 = 1, 256, 2, 96, 16
     scale = 2.0 ** -4 / math.log2(math.e)
     g = torch.Generator().manual_seed(21)
     q = torch.pow(2.0, torch.randint(-1, 2, (b, n, h, d), generator=g).float()).bfloat16()
@@ -163,6 +168,8 @@ def test_backward_that_recomputes_instead_of_using_saved_partials(shape, monkeyp
     (torch.bfloat16, 64, 32, 200, 64, 16),     # value heads narrower than query/key heads
     (torch.float16, 48, 128, 150, 40, 8),      # neither 64 nor 128; value heads wider
     (torch.bfloat16, 96, 96, 100, 512, 32),
+    (torch.bfloat16, 192, 192, 100, 64, 32),   # padded to 256
+    (torch.float32, 256, 160, 70, 512, 8),     # query/key heads of 256, narrower value heads
 ])
 def test_other_head_dimensions_and_dtypes(dtype, dqk, dv, n, w1, w2):
     """Head dimensions other than 32/64/128 (and the native 32), a value head dimension of its own, and float16 /
@@ -185,8 +192,9 @@ def test_other_head_dimensions_and_dtypes(dtype, dqk, dv, n, w1, w2):
     U.check_all(out, grads, ref_out, ref_grads, unit_variance=True)
 
 
-def test_backward_is_deterministic():
-    ins = U.make_inputs(1, 384, 2, 1, 128, seed=11)
+@pytest.mark.parametrize('d', [128, 256])
+def test_backward_is_deterministic(d):
+    ins = U.make_inputs(1, 384, 2, 1, d, seed=11)
     first = U.hip_fwd_bwd(*ins, 128, 32)
     for _ in range(2):
         again = U.hip_fwd_bwd(*ins, 128, 32)
@@ -274,6 +282,57 @@ def test_each_backward_entry_point_against_the_oracle():
     torch.cuda.synchronize()
     assert torch.equal(dq2, dq) and torch.equal(g2[1], dk2) and torch.equal(g2[3], dv2)
     assert torch.equal(g2[0], dk1) and torch.equal(g2[2], dv1)
+
+
+def test_head_dimension_256_entry_points_one_by_one():
+    """Head dimension 256 through every entry point of the C ABI: the forward without saved partials (its kernels keep
+    none), delta, sa2_bwd_dq_dkv2 on a NaN-filled workspace, sa2_bwd_dkv1, then sa2_bwd and sa2_bwd_noalloc, which must
+    give the same bits."""
+    from simplicial_attention_amd import _native
+    lib = _native.load()
+    arg = _native.tensor_arg
+    b, n, hq, hk, d, w1, w2 = 2, 210, 4, 2, 256, 70, 20
+    ins = U.make_inputs(b, n, hq, hk, d, seed=91, std=d ** -0.5)
+    ref_out, ref_lse, ref_grads = U.oracle_fwd_bwd(*ins, w1, w2)
+    q, k1, k2, v1, v2, dout = (t.cuda() for t in ins)
+    prob = _native.problem(b, n, hq, hk, d, w1, w2, True, d ** -0.5)
+    sh = torch.cuda.current_stream().cuda_stream
+    out, res = torch.full_like(q, float('nan')), torch.full_like(q, float('nan'))
+    lse = torch.full((b, hq, n), float('nan'), dtype=torch.float32, device='cuda')
+    _native.check(lib.sa2_fwd(prob, arg(q), arg(k1), arg(k2), arg(v1), arg(v2), arg(out), arg(res), lse.data_ptr(), None, sh))
+    delta = torch.full_like(lse, float('nan'))
+    _native.check(lib.sa2_bwd_delta(prob, arg(out), arg(res), arg(dout), delta.data_ptr(), sh))
+    torch.cuda.synchronize()
+    assert U.compare('out', out, ref_out)['bad'] == 0
+    assert torch.allclose(lse.cpu(), ref_lse, atol=2e-2, rtol=1e-2)
+    assert torch.allclose(delta.cpu(), (ref_out * ins[5].float()).sum(-1).transpose(1, 2), atol=2e-2, rtol=1e-2)
+    ws_bytes = lib.sa2_bwd_workspace_bytes(prob)
+    ws = torch.full((ws_bytes,), 0xFF, dtype=torch.uint8, device='cuda')
+    dq, dk2, dv2 = torch.full_like(q, float('nan')), torch.full_like(k2, float('nan')), torch.full_like(v2, float('nan'))
+    _native.check(lib.sa2_bwd_dq_dkv2(prob, arg(q), arg(k1), arg(k2), arg(v1), arg(v2), arg(dout), lse.data_ptr(), delta.data_ptr(),
+                                      None, arg(dq), arg(dk2), arg(dv2), ws.data_ptr(), ws_bytes, sh))
+    dk1, dv1 = torch.full_like(k1, float('nan')), torch.full_like(v1, float('nan'))
+    _native.check(lib.sa2_bwd_dkv1(prob, arg(q), arg(k1), arg(k2), arg(v1), arg(v2), arg(dout), lse.data_ptr(), delta.data_ptr(),
+                                   arg(dk1), arg(dv1), sh))
+    torch.cuda.synchronize()
+    for name, got, ref in zip(U.NAMES[1:], (dq, dk1, dk2, dv1, dv2), ref_grads):
+        row = U.compare(name, got, ref)
+        print('  ', row, flush=True)
+        assert row['bad'] == 0 and row['rel_fro'] <= 1e-2, row
+    for entry in ('sa2_bwd', 'sa2_bwd_noalloc'):
+        g = [torch.full_like(q, float('nan'))] + [torch.full_like(k1, float('nan')) for _ in range(4)]
+        if entry == 'sa2_bwd':
+            ws.fill_(0xFF)
+            delta2 = torch.full_like(lse, float('nan'))
+            _native.check(lib.sa2_bwd(prob, arg(q), arg(k1), arg(k2), arg(v1), arg(v2), arg(out), arg(res), arg(dout), lse.data_ptr(), None,
+                                      delta2.data_ptr(), *(arg(t) for t in g), ws.data_ptr(), ws_bytes, sh))
+        else:
+            assert lib.sa2_bwd_noalloc_scratch_bytes(prob) <= 64 << 20
+            _native.check(lib.sa2_bwd_noalloc(prob, arg(q), arg(k1), arg(k2), arg(v1), arg(v2), arg(out), arg(res), arg(dout), lse.data_ptr(),
+                                              None, *(arg(t) for t in g), sh))
+        torch.cuda.synchronize()
+        for got, want in zip(g, (dq, dk1, dk2, dv1, dv2)):
+            assert torch.equal(got, want), entry
 
 
 @pytest.mark.gpu
