@@ -47,21 +47,20 @@ __device__ __forceinline__ void wide_piece(int tid, int n, int &row, int &col) {
     col = (x % WideCfg<D>::PPR) * 16;
 }
 
-// rows row0 .. row0 + 31 of a (seq, dim) matrix into a swizzled LDS tile (rows outside the sequence are replaced by
-// the nearest row inside: whatever they meet is masked)
+// this thread's pieces into a swizzled LDS tile
 template <int D>
-__device__ __forceinline__ void wide_stage(char *tile, const char *g, int64_t sn, int row0, int N, int tid) {
+__device__ __forceinline__ void wide_store(char *tile, const u32x4 (&src)[WideCfg<D>::NP], int tid) {
 #pragma unroll
     for (int n = 0; n < WideCfg<D>::NP; ++n) {
         int row, col;
         wide_piece<D>(tid, n, row, col);
-        int rr = row0 + row;
-        rr = rr < 0 ? 0 : (rr < N ? rr : N - 1);
-        *reinterpret_cast<u32x4 *>(tile + swz_store_off<D>(row, col)) = ld_global16(g + (int64_t)rr * sn + col);
+        *reinterpret_cast<u32x4 *>(tile + swz_store_off<D>(row, col)) = src[n];
     }
 }
 
-// this thread's pieces of rows row0 .. row0 + 31, kept in registers
+// this thread's pieces of rows row0 .. row0 + 31 of a (seq, dim) matrix, into registers (rows outside the sequence
+// are replaced by the nearest row inside: whatever they meet is masked).  The kernels fetch a tile one step ahead,
+// so that the memory latency passes behind the step's MFMAs.
 template <int D>
 __device__ __forceinline__ void wide_pieces(u32x4 (&dst)[WideCfg<D>::NP], const char *g, int64_t sn, int row0, int N, int tid) {
 #pragma unroll
@@ -74,20 +73,16 @@ __device__ __forceinline__ void wide_pieces(u32x4 (&dst)[WideCfg<D>::NP], const 
     }
 }
 
-// operand tile: row r = bf16(x_r * y_{r - dlt} * c), x from registers, y rows row0 - dlt + r from global memory
+// operand tile: piece = bf16(x * y * c), x and y from registers (y: the pieces of rows row0 - dlt .. row0 - dlt + 31)
 template <int D>
-__device__ __forceinline__ void wide_build(char *tile, const u32x4 (&x)[WideCfg<D>::NP], const char *yg, int64_t sn, int row0, int dlt, int N,
-                                           float c, int tid) {
+__device__ __forceinline__ void wide_build(char *tile, const u32x4 (&x)[WideCfg<D>::NP], const u32x4 (&y)[WideCfg<D>::NP], float c, int tid) {
 #pragma unroll
     for (int n = 0; n < WideCfg<D>::NP; ++n) {
         int row, col;
         wide_piece<D>(tid, n, row, col);
-        int rr = row0 + row - dlt;
-        rr = rr < 0 ? 0 : (rr < N ? rr : N - 1);
-        const u32x4 y = ld_global16(yg + (int64_t)rr * sn + col);
         u32x4 a;
 #pragma unroll
-        for (int w = 0; w < 4; ++w) a[w] = pack_bf16(bf16_lo(x[n][w]) * c * bf16_lo(y[w]), bf16_hi(x[n][w]) * c * bf16_hi(y[w]));
+        for (int w = 0; w < 4; ++w) a[w] = pack_bf16(bf16_lo(x[n][w]) * c * bf16_lo(y[n][w]), bf16_hi(x[n][w]) * c * bf16_hi(y[n][w]));
         *reinterpret_cast<u32x4 *>(tile + swz_store_off<D>(row, col)) = a;
     }
 }
@@ -157,16 +152,28 @@ __global__ __launch_bounds__(256) void fwd_wide_kernel(KParams p) {
 #pragma unroll
     for (int db = 0; db < DB; ++db) O[db] = zero16();
 
+    // fetched one step ahead: the k2 rows of the next offset, the K1 / V1 rows of the next tile
+    u32x4 ny[C::NP], nk[C::NP], nv[C::NP];
+    wide_pieces<D>(ny, k2g, p.k2.sn, i0, N, tid);
+    wide_pieces<D>(nk, k1g, p.k1.sn, 32 * t_lo, N, tid);
+    wide_pieces<D>(nv, v1g, p.v1.sn, 32 * t_lo, N, tid);
+
     for (int dlt = 0; dlt < nd; ++dlt) {
         __syncthreads();                                 // the operand tile of the offset before is no longer read
-        wide_build<D>(tA, qp, k2g, p.k2.sn, i0, dlt, N, p.scale_log2e, tid);
+        wide_build<D>(tA, qp, ny, p.scale_log2e, tid);
+        wide_pieces<D>(ny, k2g, p.k2.sn, i0 - dlt - 1, N, tid);
 #pragma unroll
         for (int db = 0; db < DB; ++db) T[db] = zero16();
         const bool col_ok = row_ok && i - dlt >= 0;
         for (int t = t_lo; t <= t_hi; ++t) {
             __syncthreads();                             // the tiles of the step before are no longer read
-            wide_stage<D>(tK, k1g, p.k1.sn, 32 * t, N, tid);
-            wide_stage<D>(tV, v1g, p.v1.sn, 32 * t, N, tid);
+            wide_store<D>(tK, nk, tid);
+            wide_store<D>(tV, nv, tid);
+            {
+                const int tn = t < t_hi ? t + 1 : t_lo;
+                wide_pieces<D>(nk, k1g, p.k1.sn, 32 * tn, N, tid);
+                wide_pieces<D>(nv, v1g, p.v1.sn, 32 * tn, N, tid);
+            }
             __syncthreads();
             f32x16 X = zero16();
 #pragma unroll
@@ -296,17 +303,31 @@ __global__ __launch_bounds__(256) void bwd_wide_q_kernel(KParams p, float *ws, i
 #pragma unroll
     for (int db = 0; db < DB; ++db) dQ[db] = zero16();
 
+    // fetched one step ahead: the k2 / v2 rows of the next offset, the K1 / V1 rows of the next tile
+    u32x4 nyk[C::NP], nyv[C::NP], nk[C::NP], nv[C::NP];
+    wide_pieces<D>(nyk, k2g, p.k2.sn, i0, N, tid);
+    wide_pieces<D>(nyv, v2g, p.v2.sn, i0, N, tid);
+    wide_pieces<D>(nk, k1g, p.k1.sn, 32 * t_lo, N, tid);
+    wide_pieces<D>(nv, v1g, p.v1.sn, 32 * t_lo, N, tid);
+
     for (int dlt = 0; dlt < nd; ++dlt) {
         __syncthreads();      // operand tiles free; the rows this offset adds to were written at least one barrier ago
-        wide_build<D>(tA, qp, k2g, p.k2.sn, i0, dlt, N, p.scale_log2e, tid);
-        wide_build<D>(tB, dop, v2g, p.v2.sn, i0, dlt, N, 1.f, tid);
+        wide_build<D>(tA, qp, nyk, p.scale_log2e, tid);
+        wide_build<D>(tB, dop, nyv, 1.f, tid);
+        wide_pieces<D>(nyk, k2g, p.k2.sn, i0 - dlt - 1, N, tid);
+        wide_pieces<D>(nyv, v2g, p.v2.sn, i0 - dlt - 1, N, tid);
 #pragma unroll
         for (int db = 0; db < DB; ++db) G[db] = T[db] = zero16();
         const bool col_ok = row_ok && i - dlt >= 0;
         for (int t = t_lo; t <= t_hi; ++t) {
             __syncthreads();
-            wide_stage<D>(tK, k1g, p.k1.sn, 32 * t, N, tid);
-            wide_stage<D>(tV, v1g, p.v1.sn, 32 * t, N, tid);
+            wide_store<D>(tK, nk, tid);
+            wide_store<D>(tV, nv, tid);
+            {
+                const int tn = t < t_hi ? t + 1 : t_lo;
+                wide_pieces<D>(nk, k1g, p.k1.sn, 32 * tn, N, tid);
+                wide_pieces<D>(nv, v1g, p.v1.sn, 32 * tn, N, tid);
+            }
             __syncthreads();
             f32x16 X = zero16(), Y = zero16();
 #pragma unroll
@@ -432,10 +453,16 @@ __global__ __launch_bounds__(256) void bwd_wide_kv_kernel(KParams p) {
                 lse_s[tid] = p.lse[srow] * kLog2e;
                 del_s[tid] = p.delta[srow];
             }
+            // (fetched one offset ahead: the k2 / v2 rows of the next offset)
+            u32x4 nyk[C::NP], nyv[C::NP];
+            wide_pieces<D>(nyk, k2g, p.k2.sn, i0, N, tid);
+            wide_pieces<D>(nyv, v2g, p.v2.sn, i0, N, tid);
             for (int dlt = 0; dlt < nd; ++dlt) {
                 __syncthreads();                         // operand tiles and exchange areas free
-                wide_build<D>(tA, qp, k2g, p.k2.sn, i0, dlt, N, p.scale_log2e, tid);
-                wide_build<D>(tB, dop, v2g, p.v2.sn, i0, dlt, N, 1.f, tid);
+                wide_build<D>(tA, qp, nyk, p.scale_log2e, tid);
+                wide_build<D>(tB, dop, nyv, 1.f, tid);
+                wide_pieces<D>(nyk, k2g, p.k2.sn, i0 - dlt - 1, N, tid);
+                wide_pieces<D>(nyv, v2g, p.v2.sn, i0 - dlt - 1, N, tid);
                 __syncthreads();
                 // S[i][j], dP[i][j]: register rr of this lane is query row i0 + 8 (rr / 4) + 4 hf + rr % 4, the lane's column is key row j
                 f32x16 X = zero16(), Y = zero16();
