@@ -24,9 +24,10 @@
 // v2_{i-dlt} * T * 2^(M - Mc) (formed in place in T first) in eight barrier-separated phases; in phase ph wave w owns the
 // d-slice (w + ph) mod 8, so concurrent waves never touch the same element and every element
 // sees its additions in a fixed order (bitwise reproducible, no atomics).
-// The k2/v2 rows live in a 64-row circular LDS buffer (row k in slot (k - i0) mod 64): a round
-// needs 39 of them and the 8 rows that the next round adds are fetched while the round's results
-// are added to the shared accumulator.
+// The k2/v2 rows live in a 64-row circular LDS buffer (row k in slot (k - i0) mod 64), filled before the first round
+// with the rows k - i0 = -32 .. 31, which is all that second windows up to 32 ever read; a round needs 39 rows, and
+// from the fourth round on the 8 rows that the next round adds are fetched while the round's results are added to
+// the shared accumulator.
 #pragma once
 
 #include <type_traits>
@@ -59,6 +60,8 @@ struct FwdCfg {
     // to 128 registers (a few spills outside the step's MFMA blocks) so that two workgroups share a CU, which is worth
     // 20 % at D = 64; D = 32 fits by itself
     static constexpr int WPE = D == 128 ? 2 : 4;
+    // fragments in flight per operand and chain (at D = 128 four of the eight: a rolling window)
+    static constexpr int FW = KS < 4 ? KS : 4;
     static constexpr int QS = RING + ACC + 2 * EXCH;
     static constexpr int QPITCH = QF ? D * 4 + 16 : tile_pitch<D>();
     static constexpr int KSLOTS = 64;                 // circular k2 / v2 rows
@@ -174,11 +177,12 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(FwdCfg<D>::
                 *reinterpret_cast<u32x4 *>(lds + C::QS + row * C::QPITCH + col) = fq;
             }
         }
-        for (int x = tid; x < 39 * PPR; x += 512) {
+        // rows k - i0 = -32 .. 31 fill the 64 slots: the first four rounds find their rows here
+        for (int x = tid; x < 64 * PPR; x += 512) {
             const int row = x / PPR, col = (x % PPR) * 16;
-            int kk2 = i0 - 7 + row;
+            int kk2 = i0 - 32 + row;
             kk2 = kk2 < 0 ? 0 : (kk2 < N ? kk2 : N - 1);
-            const int slot = (row - 7) & 63;
+            const int slot = (row - 32) & 63;
             *reinterpret_cast<u32x4 *>(lds + C::K2S + slot * PITCH + col) = ld_global16(k2g + (int64_t)kk2 * p.k2.sn + col);
             *reinterpret_cast<u32x4 *>(lds + C::V2S + slot * PITCH + col) = ld_global16(v2g + (int64_t)kk2 * p.v2.sn + col);
         }
@@ -195,7 +199,9 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(FwdCfg<D>::
         for (int e = 0; e < 4; ++e) mp[e] = ((unsigned)(rel - (8 * qq + e)) < (unsigned)p.w1) ? 0.f : -INFINITY;
         *reinterpret_cast<float4 *>(lds + C::MASKS + tab * C::MASK + qq * 1024 + ln * 16) = m4;
     }
-    // the 8 rows that round r + 1 adds (k - i0 = -8r - 15 .. -8r - 8), one 16-byte piece per thread
+    // the 8 rows that round r + 1 adds (k - i0 = -8r - 15 .. -8r - 8), one 16-byte piece per thread; only rounds
+    // beyond the fourth add rows that the prologue has not staged
+    auto adds_rows = [&](int r) { return r + 1 < R && r + 1 >= 4; };
     const bool row_stager = tid < 2 * 8 * PPR;
     const int rs_sel = tid / (8 * PPR), rs_row = (tid / PPR) % 8, rs_col = (tid % PPR) * 16;
     u32x4 st_r = {0u, 0u, 0u, 0u};
@@ -221,8 +227,11 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(FwdCfg<D>::
     };
     f32x16 T[DT];
     u32x4 A[KS];
-    u32x4 kf[KS];              // K1 fragments of the step about to run (requested at the end of the step before, or at the round's start)
-    u32x2 vf[DT][2][2];        // V1 fragments of the running step (requested when its logit chain has been issued)
+    // Fragments travel through rolling windows of FW register sets: fragment f of a chain sits in set f % FW and is
+    // requested FW MFMAs before its use, the first FW fragments of a chain along the tail of the chain before
+    constexpr int FW = C::FW;
+    u32x4 kf[FW];              // K1 fragments (row fragments)
+    u32x2 vf[FW][2];           // V1 fragments (two transposed reads each)
     float M = 0.f;             // softmax reference of the row (log2 domain); meaningless while `fresh`
     bool fresh = true;         // the row has not met an attended entry yet
     float l = 0.f;             // this lane's part of the row sum, relative to M
@@ -308,35 +317,42 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(FwdCfg<D>::
         auto load_kf = [&](int buf_off) {
             const char *kbase = lds + buf_off + k_lane;
 #pragma unroll
-            for (int kk = 0; kk < KS; ++kk) kf[kk] = ld_lds16(kbase + C::RT::row_imm(kk));
+            for (int kk = 0; kk < FW; ++kk) kf[kk] = ld_lds16(kbase + C::RT::row_imm(kk));
         };
         // The fragment reads of a step sit between its MFMAs, a scheduling fence behind every MFMA and its reads
         // keeps them there: the V1 fragments of the tile along its logit chain, the K1 fragments of the next tile
         // along the value chain.
         // (the K1 fragments behind the round's last tile are those of the next round's first tile: the ring runs on)
+        auto read_vf = [&](const char *vbase, int f) {
+            const int k2s = f / DT, dt = f % DT;
+            vf[f % FW][0] = lds_read_tr<D, 0>(vbase + C::RT::tr_imm(16 * k2s, 32 * dt), 0, 0);
+            vf[f % FW][1] = lds_read_tr<D, 0>(vbase + C::RT::tr_imm(16 * k2s + 8, 32 * dt), 0, 0);
+        };
         auto value_products = [&](const u32x4 (&pb)[2]) {
             const char *kbase = lds + b_nxt + k_lane;
+            const char *vbase = lds + b_cur + v_lane;
 #pragma unroll
-            for (int m = 0; m < 2 * DT; ++m) {
+            for (int m = 0; m < KS; ++m) {
                 const int k2s = m / DT, dt = m % DT;
-                u32x4 v = {vf[dt][k2s][0][0], vf[dt][k2s][0][1], vf[dt][k2s][1][0], vf[dt][k2s][1][1]};
+                u32x4 v = {vf[m % FW][0][0], vf[m % FW][0][1], vf[m % FW][1][0], vf[m % FW][1][1]};
                 T[dt] = mfma32(v, pb[k2s], T[dt]);
-                kf[m] = ld_lds16(kbase + C::RT::row_imm(m));
+                if (m + FW < KS) read_vf(vbase, m + FW);
+                if (m >= KS - FW) kf[m - (KS - FW)] = ld_lds16(kbase + C::RT::row_imm(m - (KS - FW)));
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
         auto logit_chain = [&](f32x16 &X, auto loads_tag) {
+            const char *kbase = lds + b_cur + k_lane;
             const char *vbase = lds + b_cur + v_lane;
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int kk = 0; kk < KS; ++kk) {
-                X = mfma32(kf[kk], A[kk], X);
+                X = mfma32(kf[kk % FW], A[kk], X);
                 if constexpr (decltype(loads_tag)::value) {
                     if (kk == 0) issue_loads();
                 }
-                const int k2s = kk / DT, dt = kk % DT;
-                vf[dt][k2s][0] = lds_read_tr<D, 0>(vbase + C::RT::tr_imm(16 * k2s, 32 * dt), 0, 0);
-                vf[dt][k2s][1] = lds_read_tr<D, 0>(vbase + C::RT::tr_imm(16 * k2s + 8, 32 * dt), 0, 0);
+                if (kk + FW < KS) kf[kk % FW] = ld_lds16(kbase + C::RT::row_imm(kk + FW));
+                if (kk >= KS - FW) read_vf(vbase, kk - (KS - FW));
                 __builtin_amdgcn_sched_barrier(0);
             }
         };
@@ -452,7 +468,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(FwdCfg<D>::
 
         // ---- round end: agree on the common reference, add v2 * T into the shared rows
         {
-            if (r + 1 < R) issue_rows(r);      // the rows that the next round adds arrive behind the phases below
+            if (adds_rows(r)) issue_rows(r);   // the rows that the next round adds arrive behind the phases below
             if (hf == 0) xm[wave * 32 + c] = fresh ? -INFINITY : M;
             __syncthreads();
             float Mn = Mc;
@@ -506,7 +522,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(FwdCfg<D>::
             for (int ph = 0; ph < 8; ++ph) {
                 constexpr int NS = 2 * DT;
                 if (NS == 8 || ph / NS == wave / NS) with_slice<NS>(wave + ph, [&](auto tag) { add_slice(tag, ph % NS == 0 && (NS == 8 || wave / NS == 0)); });
-                if (ph == 7 && r + 1 < R) write_rows(r);    // (their slots are not in use in this round)
+                if (ph == 7 && adds_rows(r)) write_rows(r);  // (their slots are not in use in this round)
                 __syncthreads();
             }
         }
