@@ -108,15 +108,18 @@ def cpu_baseline(N, D, w1, w2, slices, runs=3, naive_runs=5):
     }
 
 
+# the sources that the kernels of head dimensions 32, 64 and 128 are built from (the kernels whose HBM traffic is stored)
+MEASURED_KERNEL_SOURCES = ('sa2_common.hpp', 'sa2_lds.hpp', 'sa2_fwd.hpp', 'sa2_bwd.hpp', 'sa2_bwd_q.hpp', 'sa2_bwd_kv8.hpp')
+
+
 def source_digest():
-    """sha256 over the kernel sources: ties a stored counter measurement to the code it was taken on."""
-    import glob
+    """sha256 over the sources of the measured kernels: ties a stored counter measurement to the code it was taken on."""
     import hashlib
     h = hashlib.sha256()
     csrc = os.path.join(ROOT, 'simplicial_attention_amd', 'csrc')
-    for f in sorted(glob.glob(os.path.join(csrc, '*.hpp')) + glob.glob(os.path.join(csrc, '*.hip'))):
-        h.update(os.path.basename(f).encode())
-        h.update(open(f, 'rb').read())
+    for name in MEASURED_KERNEL_SOURCES:
+        h.update(name.encode())
+        h.update(open(os.path.join(csrc, name), 'rb').read())
     return h.hexdigest()[:16]
 
 
@@ -235,6 +238,31 @@ def mfma_mix_rates(iters=2048, workgroups=1024):
             tf = workgroups * 8 * iters * 16 * 32768 / (best * 1e-3) / 1e12
             res['%s_operands__%s' % (dname, mname)] = {'tflops': round(tf, 1), 'frac_of_nominal_peak': round(tf / PEAK_BF16_TFLOPS, 4),
                                                         'shader_clock_mhz': round(100.0 * int(c[0]) / max(int(c[1]), 1), 0)}
+    return res
+
+
+def vendor_gemm_rates(n=8192, iters=10):
+    """The same question put to the vendor's GEMM: torch.matmul of two n x n bf16 matrices (hipBLASLt) on random,
+    all-zero and all-one operands.  Operands that do not toggle run faster on the same code."""
+    import torch
+    dev = torch.device('cuda:0')
+    g = torch.Generator(device='cpu').manual_seed(11)
+    res = {}
+    for name in ('random', 'zeros', 'ones'):
+        if name == 'random':
+            a, b_ = (torch.randn(n, n, generator=g).bfloat16().to(dev) for _ in range(2))
+        else:
+            a, b_ = (torch.full((n, n), 0.0 if name == 'zeros' else 1.0, dtype=torch.bfloat16, device=dev) for _ in range(2))
+        for _ in range(3):
+            torch.matmul(a, b_)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            torch.matmul(a, b_)
+        torch.cuda.synchronize()
+        t = (time.perf_counter() - t0) / iters
+        tf = 2 * n ** 3 / t / 1e12
+        res['%s_operands' % name] = {'ms': round(t * 1e3, 3), 'tflops': round(tf, 1), 'frac_of_nominal_peak': round(tf / PEAK_BF16_TFLOPS, 4)}
     return res
 
 
@@ -398,7 +426,7 @@ def main():
         print(json.dumps(time_module_cfg2()))
         return
     if args.only == 'mfma_mix':
-        print(json.dumps(mfma_mix_rates()))
+        print(json.dumps({'instruction_mix_loop': mfma_mix_rates(), 'torch_matmul_bf16_8192': vendor_gemm_rates()}))
         return
     if args.only == 'copy':
         # plain device copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters

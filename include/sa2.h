@@ -40,8 +40,10 @@ extern "C" {
 #endif
 
 /* 101: saved->t is kept in blocks of 32 rows (sa2_saved_t_bytes), the workspace rules of sa2_bwd_workspace_bytes*
- * cover the split key slabs, sa2_bwd checks every size before its first launch */
-#define SA2_VERSION 101
+ * cover the split key slabs, sa2_bwd checks every size before its first launch
+ * 102: dim_head 256 (its kernels keep no forward partials: the sa2_saved_*_bytes queries return 0 and a non-NULL
+ * `saved` is refused) */
+#define SA2_VERSION 102
 
 typedef enum sa2_status {
     SA2_OK = 0,
@@ -60,7 +62,7 @@ typedef struct sa2_problem {
     int32_t seq_len;
     int32_t heads;      /* query heads */
     int32_t kv_heads;   /* key/value heads, divides heads */
-    int32_t dim_head;   /* 32, 64 or 128 */
+    int32_t dim_head;   /* 32, 64, 128 or 256 */
     int32_t w1;         /* window of the first key/value set  (reference default 512) */
     int32_t w2;         /* window of the second key/value set (reference default 32), any value >= 1 */
     int32_t causal;     /* must be 1 */
@@ -84,13 +86,14 @@ typedef struct sa2_tensor {
  *      for the offset d = i - k, x = scaled logit * log2(e)
  *   m  fp32 [batch][heads][w2][seq_len]:            the reference m of that sum
  * With them dV2[k] = sum_d dO[k+d] * T[d,k+d] * 2^(m - lse*log2e) needs no contraction
- * in the backward.  Sizes: sa2_saved_t_bytes(), sa2_saved_m_bytes().  t 16-byte aligned. */
+ * in the backward.  Sizes: sa2_saved_t_bytes(), sa2_saved_m_bytes().  t 16-byte aligned.
+ * dim_head 256 keeps no partials: both sizes are 0 and its calls take saved = NULL. */
 typedef struct sa2_saved {
     void  *t;
     float *m;
 } sa2_saved;
 
-int64_t sa2_saved_t_bytes(const sa2_problem *prob);   /* -1 if the problem is invalid */
+int64_t sa2_saved_t_bytes(const sa2_problem *prob);   /* -1 if the problem is invalid, 0 if its kernels keep no partials */
 int64_t sa2_saved_m_bytes(const sa2_problem *prob);
 
 /* Library version (SA2_VERSION of the build). */
@@ -99,7 +102,7 @@ int sa2_version(void);
 /* Message of the last failing call on this thread ("" if none). */
 const char *sa2_last_error(void);
 
-/* 1 if the kernels cover this configuration (dim_head 32, 64 or 128, any w1 >= 1 and w2 >= 1, bf16),
+/* 1 if the kernels cover this configuration (dim_head 32, 64, 128 or 256, any w1 >= 1 and w2 >= 1, bf16),
  * else 0.  Replaces the silent limits of the reference (HEAD_DIM fixed to 64, w2 <= 32:
  * triton_two_simplicial_attention.py:51,291,508,586). */
 int sa2_supported(int32_t dim_head, int32_t w1, int32_t w2, int32_t dtype);

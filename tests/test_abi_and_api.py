@@ -33,7 +33,7 @@ def test_every_declared_symbol_is_exported(lib):
     assert set(names) == set(_native.EXPORTS)
     for name in names:
         assert getattr(lib, name) is not None
-    assert lib.sa2_version() == 101
+    assert lib.sa2_version() == 102
 
 
 def test_supported_matrix(lib):
