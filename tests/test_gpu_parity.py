@@ -49,12 +49,12 @@ def test_fwd_bwd_matches_oracle(b, n, hq, hk, d, w1, w2, unit_variance):
     U.check_all(out, grads, ref_out, ref_grads, unit_variance=unit_variance)
 
 
-def _random_shapes(count, seed=1234):
+def _random_shapes(count, seed=1234, dims=(32, 64, 128)):
     import random
     rng = random.Random(seed)
     shapes = []
     for _ in range(count):
-        d = rng.choice([32, 64, 128])
+        d = rng.choice(list(dims))
         hk = rng.choice([1, 2])
         hq = hk * rng.choice([1, 2])
         n = rng.choice([rng.randint(1, 40), rng.randint(33, 130), rng.randint(131, 420)])
@@ -68,6 +68,16 @@ def _random_shapes(count, seed=1234):
 def test_seeded_random_shapes(b, n, hq, hk, d, w1, w2):
     """A seeded draw of sequence lengths, windows, head counts and head dimensions (ragged tiles, windows
     shorter and longer than the sequence, one to ten offset rounds, grouped heads)."""
+    print(f'\ncase b={b} n={n} hq={hq} hk={hk} d={d} w1={w1} w2={w2}', flush=True)
+    ins = U.make_inputs(b, n, hq, hk, d, seed=n * 7 + w1 * 3 + w2, std=d ** -0.5)
+    ref_out, _, ref_grads = U.oracle_fwd_bwd(*ins, w1, w2)
+    out, grads = U.hip_fwd_bwd(*ins, w1, w2)
+    U.check_all(out, grads, ref_out, ref_grads)
+
+
+@pytest.mark.parametrize('b,n,hq,hk,d,w1,w2', _random_shapes(10, seed=4321, dims=(256,)))
+def test_seeded_random_shapes_head_dimension_256(b, n, hq, hk, d, w1, w2):
+    """The same draw for the kernels of head dimension 256."""
     print(f'\ncase b={b} n={n} hq={hq} hk={hk} d={d} w1={w1} w2={w2}', flush=True)
     ins = U.make_inputs(b, n, hq, hk, d, seed=n * 7 + w1 * 3 + w2, std=d ** -0.5)
     ref_out, _, ref_grads = U.oracle_fwd_bwd(*ins, w1, w2)
