@@ -60,8 +60,9 @@ struct FwdCfg {
     // to 128 registers (a few spills outside the step's MFMA blocks) so that two workgroups share a CU, which is worth
     // 20 % at D = 64; D = 32 fits by itself
     static constexpr int WPE = D == 128 ? 2 : 4;
-    // fragments in flight per operand and chain (at D = 128 four of the eight: a rolling window)
-    static constexpr int FW = KS < 4 ? KS : 4;
+    // fragments in flight per operand and chain: a rolling window of four of the eight at D = 128; two of the four at
+    // D = 64, where four waves per SIMD cover the latency and the registers are the scarcer resource
+    static constexpr int FW = D == 64 ? 2 : (KS < 4 ? KS : 4);
     static constexpr int QS = RING + ACC + 2 * EXCH;
     static constexpr int QPITCH = QF ? D * 4 + 16 : tile_pitch<D>();
     static constexpr int KSLOTS = 64;                 // circular k2 / v2 rows
