@@ -213,8 +213,10 @@ int sa2_fwd(const sa2_problem *prob, const sa2_tensor *q, const sa2_tensor *k1, 
         k.m_save = saved->m;
     }
     const int grid = prob->batch * prob->heads * ((prob->seq_len + 31) / 32);
-    if (prob->dim_head == kWideDimHead)
-        hipLaunchKernelGGL(sa2::fwd_wide_kernel<kWideDimHead>, dim3(grid), dim3(256), 0, s, k);
+    if (prob->dim_head == kWideDimHead) {
+        const int wgrid = prob->batch * prob->heads * ((prob->seq_len + 127) / 128);
+        hipLaunchKernelGGL(sa2::fwd_wide_kernel<kWideDimHead>, dim3(wgrid), dim3(256), 0, s, k);
+    }
     else
         SA2_FOR_DIM_HEAD(prob->dim_head, hipLaunchKernelGGL(sa2::fwd_kernel<DH>, dim3(grid), dim3(512), 0, s, k));
     return after_launch("forward");

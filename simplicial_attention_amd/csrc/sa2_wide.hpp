@@ -1,22 +1,27 @@
 // Kernels for head dimension 256: forward, dQ/dK2/dV2 and dK1/dV1.
 //
 // At D = 256 neither the logit operand (64 registers) nor a [32][D] fp32 accumulator (128 registers) leaves room
-// for the register-resident designs of the other head dimensions, so the four waves of a workgroup split the head
-// dimension instead: wave w owns the columns d = 64 w .. 64 w + 63.  Every 32 x 32 logit tile is the sum of four
+// for the two-waves-per-SIMD, register-resident designs of the other head dimensions.
+//
+//   fwd_wide_kernel     one wave per SIMD with all 512 registers: a workgroup of four waves owns four consecutive
+//                       query tiles, one per wave; a wave keeps the logit operand, the value accumulator T of the
+//                       running offset and the output sum O in registers and shares only the K1 / V1 tiles (LDS)
+//                       with the other waves.  For every offset dlt = i - k, for every tile: S^T = K1 A^T, running
+//                       softmax over all (offset, tile) pairs, T^T += V1^T P^T; at the end of an offset
+//                       O += v2_{i-dlt} * T                                      (reference: TT:58-228)
+// The backward kernels hold two accumulators per output row set and split the head dimension over the four waves of
+// a workgroup instead: wave w owns the columns d = 64 w .. 64 w + 63.  Every 32 x 32 logit tile is the sum of four
 // partial contractions (one per wave, four MFMAs each) that meet in an fp32 exchange area of LDS; every wave then
 // holds the complete tile in the MFMA's C layout, forms the same weights, and multiplies them into its own 64
-// columns of the value-side accumulators.  No MFMA is issued twice.  Operand tiles live in LDS in the swizzled
-// layout of SwzLane (written once, read as row fragments and as transposed fragments).
-//
-//   fwd_wide_kernel     owns 32 query rows: for every offset dlt = i - k, for every K1/V1 tile: S^T = K1 A^T,
-//                       running softmax over all (offset, tile) pairs, T^T += V1^T P^T; at the end of an offset
-//                       O += v2_{i-dlt} * T                                      (reference: TT:58-228)
+// columns of the accumulators.  No MFMA is issued twice.
 //   bwd_wide_q_kernel   owns 32 query rows: S, dP, dS = P (dP - delta), G^T += K1^T dS^T, T^T += V1^T P^T;
 //                       dq += k2 * G in registers, dk2 / dv2 partial rows (q * G, do * T) added to the fp32
 //                       workspace block of the tile, which dk2_dv2_combine_kernel sums (TT:515-712)
 //   bwd_wide_kv_kernel  owns 32 rows j of K1/V1: for every query tile and offset that reaches them
 //                       dV1^T += B^T P, dK1^T += A^T dS                              (TT:298-503)
 // (TT = simplicial_attention/triton_two_simplicial_attention.py of the reference.)
+// Operand tiles live in LDS in the swizzled layout of SwzLane (written once, read as row fragments and as
+// transposed fragments); tiles and rows are fetched one step ahead through registers.
 // Every sum has a fixed order: results are bitwise reproducible, there are no atomics.
 #pragma once
 
@@ -114,139 +119,189 @@ __device__ __forceinline__ void wide_pack(u32x4 (&pb)[2], const f32x16 &X) {
 }
 
 // ------------------------------------------------------------------------------------------------------------------
+// Forward, one wave per SIMD: a workgroup of four waves owns four consecutive 32-row query tiles, one per wave, and a
+// wave keeps everything of its tile in its 512 registers: the logit operand A (64), the value accumulator T of the
+// running offset (128) and the output sum O over the offsets (128).  Nothing is exchanged between waves: the
+// workgroup only shares the K1 / V1 tiles, which go through two LDS buffers (one barrier per tile step).  The waves'
+// first windows differ by one tile each: the workgroup walks the union and a wave skips what lies outside its own.
 template <int D>
-__global__ __launch_bounds__(256) void fwd_wide_kernel(KParams p) {
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void fwd_wide_kernel(KParams p) {
     using C = WideCfg<D>;
-    constexpr int DB = C::DB, KQ = C::KQ;
-    __shared__ __attribute__((aligned(16))) char lds[3 * C::TILE + C::XCH];
-    char *tA = lds, *tK = lds + C::TILE, *tV = lds + 2 * C::TILE, *xch = lds + 3 * C::TILE;
+    constexpr int KS = D / 16, DT = D / 32;
+    __shared__ __attribute__((aligned(16))) char lds[4 * C::TILE];
 
     const int N = p.N;
-    const int ntile = (N + 31) / 32;
+    const int ntile = (N + 31) / 32, ngroup = (ntile + 3) / 4;
     const int item = xcd_contiguous(blockIdx.x, gridDim.x);
-    const int tile = ntile - 1 - item % ntile;
-    const int bh = item / ntile;
+    const int grp = ngroup - 1 - item % ngroup;
+    const int bh = item / ngroup;
     const int h = bh % p.H, b = bh / p.H;
     const int hk = h / p.G;
     const int tid = threadIdx.x;
     const int wave = wave_index(), lane = tid & 63;
     const int c = lane & 31, hf = lane >> 5;
+    const int tile = 4 * grp + wave;
+    const bool tile_ok = tile < ntile;
     const int i0 = tile * 32, i = i0 + c;
     const bool row_ok = i < N;
+    const int ic = row_ok ? i : N - 1;
 
-    const char *qg = p.q.ptr + b * p.q.sb + h * p.q.sh;
+    const char *qrow = p.q.ptr + b * p.q.sb + h * p.q.sh + (int64_t)ic * p.q.sn + 16 * hf;
     const char *k1g = p.k1.ptr + b * p.k1.sb + hk * p.k1.sh;
     const char *v1g = p.v1.ptr + b * p.v1.sb + hk * p.v1.sh;
     const char *k2g = p.k2.ptr + b * p.k2.sb + hk * p.k2.sh;
     const char *v2g = p.v2.ptr + b * p.v2.sb + hk * p.v2.sh;
     const SwzLane<D> sw(lane);
 
-    u32x4 qp[C::NP];
-    wide_pieces<D>(qp, qg, p.q.sn, i0, N, tid);
+    // this wave's tiles of the first window and offsets; the workgroup's union
+    const int t_lo = (i0 - p.w1 + 1 > 0 ? i0 - p.w1 + 1 : 0) / 32, t_hi = tile;
+    const int nd = p.w2 < i0 + 32 ? p.w2 : i0 + 32;
+    const int last = (4 * grp + 3 < ntile ? 4 * grp + 3 : ntile - 1);                 // last valid tile of the group
+    const int g_lo = (128 * grp - p.w1 + 1 > 0 ? 128 * grp - p.w1 + 1 : 0) / 32, g_hi = last;
+    const int g_nd = p.w2 < 32 * last + 32 ? p.w2 : 32 * last + 32;
 
-    const int t_lo = (i0 - p.w1 + 1 > 0 ? i0 - p.w1 + 1 : 0) / 32, t_hi = i0 / 32;
-    const int nd = p.w2 < i0 + 32 ? p.w2 : i0 + 32;      // offsets that meet at least one valid k
-
-    float m = -INFINITY, l = 0.f;                        // running softmax reference (log2 domain) and this lane's part of the row sum
-    f32x16 O[DB], T[DB];
+    float M = -INFINITY, l = 0.f;            // softmax reference of the row (log2 domain; moves only when a tile's maximum
+                                             // exceeds it by more than 2^8) and this lane's part of the row sum
+    f32x16 O[DT], T[DT];
 #pragma unroll
-    for (int db = 0; db < DB; ++db) O[db] = zero16();
+    for (int dt = 0; dt < DT; ++dt) O[dt] = zero16();
 
-    // fetched one step ahead: the k2 rows of the next offset, the K1 / V1 rows of the next tile
-    u32x4 ny[C::NP], nk[C::NP], nv[C::NP];
-    wide_pieces<D>(ny, k2g, p.k2.sn, i0, N, tid);
-    wide_pieces<D>(nk, k1g, p.k1.sn, 32 * t_lo, N, tid);
-    wide_pieces<D>(nv, v1g, p.v1.sn, 32 * t_lo, N, tid);
+    u32x4 nk[C::NP], nv[C::NP];
+    wide_pieces<D>(nk, k1g, p.k1.sn, 32 * g_lo, N, tid);
+    wide_pieces<D>(nv, v1g, p.v1.sn, 32 * g_lo, N, tid);
+    int buf = 0;
 
-    for (int dlt = 0; dlt < nd; ++dlt) {
-        __syncthreads();                                 // the operand tile of the offset before is no longer read
-        wide_build<D>(tA, qp, ny, p.scale_log2e, tid);
-        wide_pieces<D>(ny, k2g, p.k2.sn, i0 - dlt - 1, N, tid);
+    for (int dlt = 0; dlt < g_nd; ++dlt) {
+        const bool off_on = tile_ok && dlt < nd;
+        const bool col_ok = off_on && row_ok && i - dlt >= 0;
+        u32x4 A[KS];
+        {
+            int kr = i - dlt;
+            kr = kr < 0 ? 0 : (kr < N ? kr : N - 1);
+            const char *k2row = k2g + (int64_t)kr * p.k2.sn + 16 * hf;
 #pragma unroll
-        for (int db = 0; db < DB; ++db) T[db] = zero16();
-        const bool col_ok = row_ok && i - dlt >= 0;
-        for (int t = t_lo; t <= t_hi; ++t) {
-            __syncthreads();                             // the tiles of the step before are no longer read
+            for (int kk = 0; kk < KS; ++kk) {
+                const u32x4 fq = ld_global16(qrow + 32 * kk), fk = ld_global16(k2row + 32 * kk);
+#pragma unroll
+                for (int w = 0; w < 4; ++w)
+                    A[kk][w] = pack_bf16(bf16_lo(fq[w]) * p.scale_log2e * bf16_lo(fk[w]), bf16_hi(fq[w]) * p.scale_log2e * bf16_hi(fk[w]));
+            }
+        }
+#pragma unroll
+        for (int dt = 0; dt < DT; ++dt) T[dt] = zero16();
+
+        for (int t = g_lo; t <= g_hi; ++t) {
+            char *tK = lds + buf * 2 * C::TILE, *tV = tK + C::TILE;
             wide_store<D>(tK, nk, tid);
             wide_store<D>(tV, nv, tid);
             {
-                const int tn = t < t_hi ? t + 1 : t_lo;
+                const int tn = t < g_hi ? t + 1 : g_lo;
                 wide_pieces<D>(nk, k1g, p.k1.sn, 32 * tn, N, tid);
                 wide_pieces<D>(nv, v1g, p.v1.sn, 32 * tn, N, tid);
             }
-            __syncthreads();
+            __syncthreads();       // the tile is complete; every wave has left the step before, whose buffer the next store takes
+            buf ^= 1;
+            if (!(off_on && t >= t_lo && t <= t_hi)) continue;
+            // (fragments through a rolling window of four: a scheduling fence behind every MFMA and its read keeps the
+            // reads spread along the chain and the live fragments at sixteen registers)
+            constexpr int FW = 4;
             f32x16 X = zero16();
+            {
+                u32x4 f[FW];
 #pragma unroll
-            for (int kq = 0; kq < KQ; ++kq) X = mfma32(sw.row_frag(tK, wave * KQ + kq), sw.row_frag(tA, wave * KQ + kq), X);
-            wide_put(xch, wave, lane, X);
-            __syncthreads();
-            X = wide_sum(xch, lane);
-            // register rr of this lane: key row j = 32 t + 8 (rr / 4) + 4 hf + rr % 4, query row i; attended iff 0 <= i - j < w1
-            const int rel = col_ok ? i - 32 * t - 4 * hf : -(1 << 30);
-            float tmax = -INFINITY;
+                for (int kk = 0; kk < FW; ++kk) f[kk] = sw.row_frag(tK, kk);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int rr = 0; rr < 16; ++rr) {
-                const bool ok = (unsigned)(rel - (8 * (rr >> 2) + (rr & 3))) < (unsigned)p.w1;
-                X[rr] = ok ? X[rr] : -INFINITY;
-                tmax = fmaxf(tmax, X[rr]);
+                for (int kk = 0; kk < KS; ++kk) {
+                    X = mfma32(f[kk % FW], A[kk], X);
+                    if (kk + FW < KS) f[kk % FW] = sw.row_frag(tK, kk + FW);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
             }
+            // register rr of this lane: key row j = 32 t + 8 (rr / 4) + 4 hf + rr % 4, query row i; attended iff 0 <= i - j < w1
+            const bool full = 32 * t + 31 <= i0 && 32 * t > i0 + 31 - p.w1 && i0 - dlt >= 0 && i0 + 31 < N;
+            if (!full) {
+                int rel = col_ok ? i - 32 * t - 4 * hf : -(1 << 30);
+                asm volatile("" : "+v"(rel));
+#pragma unroll
+                for (int rr = 0; rr < 16; ++rr) {
+                    const bool ok = (unsigned)(rel - (8 * (rr >> 2) + (rr & 3))) < (unsigned)p.w1;
+                    X[rr] = ok ? X[rr] : -INFINITY;
+                }
+            }
+            float tmax = X[0];
+#pragma unroll
+            for (int rr = 1; rr < 16; ++rr) tmax = fmaxf(tmax, X[rr]);
             {
                 auto s2 = __builtin_amdgcn_permlane32_swap(as_u32(tmax), as_u32(tmax), false, false);
                 tmax = fmaxf(as_f32(s2[0]), as_f32(s2[1]));
             }
-            const float mn = fmaxf(m, tmax);
-            const float mref = mn == -INFINITY ? 0.f : mn;
-            const float alpha = fast_exp2(m - mref);     // 0 while the row holds nothing
-            m = mn;
+            if (wave_any(tmax > M + 8.f)) {
+                // (rare after a row's first tile) the reference follows the maximum; what the row holds is rescaled
+                const float mn = fmaxf(M, tmax);
+                const float alpha = mn == -INFINITY ? 1.f : fast_exp2(M - mn);      // 0 for a row that held nothing
+                M = mn;
+                l *= alpha;
 #pragma unroll
-            for (int db = 0; db < DB; ++db)
+                for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
-                for (int rr = 0; rr < 16; ++rr) {
-                    T[db][rr] *= alpha;
-                    O[db][rr] *= alpha;
-                }
-            float ls = l * alpha;
+                    for (int rr = 0; rr < 16; ++rr) {
+                        T[dt][rr] *= alpha;
+                        O[dt][rr] *= alpha;
+                    }
+            }
+            const float mref = M == -INFINITY ? 0.f : M;
+            float ls = l;
+            u32x4 pb[2];
 #pragma unroll
-            for (int rr = 0; rr < 16; ++rr) {
-                X[rr] = fast_exp2(X[rr] - mref);
-                ls += X[rr];
+            for (int rr = 0; rr < 16; rr += 2) {
+                const float e0 = fast_exp2(X[rr] - mref), e1 = fast_exp2(X[rr + 1] - mref);
+                ls += e0 + e1;
+                pb[rr >> 3][(rr & 7) >> 1] = pack_bf16(e0, e1);
             }
             l = ls;
-            u32x4 pb[2];
-            wide_pack(pb, X);
+            {
+                u32x4 f[FW];
 #pragma unroll
-            for (int db = 0; db < DB; ++db)
+                for (int m = 0; m < FW; ++m) f[m] = sw.tr_frag(tV, m / DT, m % DT);
+                __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-                for (int k2s = 0; k2s < 2; ++k2s) T[db] = mfma32(sw.tr_frag(tV, k2s, wave * DB + db), pb[k2s], T[db]);
+                for (int m = 0; m < 2 * DT; ++m) {
+                    T[m % DT] = mfma32(f[m % FW], pb[m / DT], T[m % DT]);
+                    if (m + FW < 2 * DT) f[m % FW] = sw.tr_frag(tV, (m + FW) / DT, (m + FW) % DT);
+                    __builtin_amdgcn_sched_barrier(0);
+                }
+            }
         }
-        // O += v2_{i - dlt} * T (lanes without a valid k hold T = 0)
-        int kr = i - dlt;
-        kr = kr < 0 ? 0 : (kr < N ? kr : N - 1);
-        fma_row<DB>(O, T, v2g + (int64_t)kr * p.v2.sn + (wave * C::DQ + 16 * hf) * 2);
+        // O += v2_{i - dlt} * T (a lane without a valid k holds T = 0)
+        if (off_on) {
+            int kr = i - dlt;
+            kr = kr < 0 ? 0 : (kr < N ? kr : N - 1);
+            fma_row<DT>(O, T, v2g + (int64_t)kr * p.v2.sn + 16 * hf * 2);
+        }
     }
 
     auto s2 = __builtin_amdgcn_permlane32_swap(as_u32(l), as_u32(l), false, false);
     const float L = as_f32(s2[0]) + as_f32(s2[1]);
-    if (!row_ok) return;
+    if (!row_ok || !tile_ok) return;
     const float inv = 1.f / L;
-    const int col0 = (wave * C::DQ + 16 * hf) * 2;
-    char *orow = p.o.ptr + b * p.o.sb + (int64_t)i * p.o.sn + h * p.o.sh + col0;
-    char *rrow = p.o_lo.ptr ? p.o_lo.ptr + b * p.o_lo.sb + (int64_t)i * p.o_lo.sn + h * p.o_lo.sh + col0 : nullptr;
+    char *orow = p.o.ptr + b * p.o.sb + (int64_t)i * p.o.sn + h * p.o.sh + 16 * hf * 2;
+    char *rrow = p.o_lo.ptr ? p.o_lo.ptr + b * p.o_lo.sb + (int64_t)i * p.o_lo.sn + h * p.o_lo.sh + 16 * hf * 2 : nullptr;
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
+    for (int dt = 0; dt < DT; ++dt)
 #pragma unroll
         for (int half = 0; half < 2; ++half) {
             u32x4 ov, rv;
 #pragma unroll
             for (int w = 0; w < 4; ++w) {
-                const float a = O[db][8 * half + 2 * w] * inv, bb = O[db][8 * half + 2 * w + 1] * inv;
+                const float a = O[dt][8 * half + 2 * w] * inv, bb = O[dt][8 * half + 2 * w + 1] * inv;
                 ov[w] = pack_bf16(a, bb);
                 rv[w] = pack_bf16(a - bf16_lo(ov[w]), bb - bf16_hi(ov[w]));
             }
-            st_global16(orow + db * 64 + half * 16, ov);
-            if (rrow) st_global16(rrow + db * 64 + half * 16, rv);
+            st_global16(orow + dt * 64 + half * 16, ov);
+            if (rrow) st_global16(rrow + dt * 64 + half * 16, rv);
         }
-    if (wave == 0 && hf == 0) p.lse[((int64_t)b * p.H + h) * N + i] = (m + __builtin_amdgcn_logf(L)) * kLn2;
+    if (hf == 0) p.lse[((int64_t)b * p.H + h) * N + i] = (M + __builtin_amdgcn_logf(L)) * kLn2;
 }
 
 // ------------------------------------------------------------------------------------------------------------------
