@@ -97,25 +97,28 @@ __device__ __forceinline__ void wide_put(char *xch, int wave, int lane, const f3
     for (int r4 = 0; r4 < 4; ++r4)
         *reinterpret_cast<float4 *>(xch + wave * 4096 + r4 * 1024 + lane * 16) = make_float4(X[4 * r4], X[4 * r4 + 1], X[4 * r4 + 2], X[4 * r4 + 3]);
 }
-// sum of the four waves' partial tiles, in wave order (every wave forms the same bits)
-__device__ __forceinline__ f32x16 wide_sum(const char *xch, int lane) {
-    f32x16 X = zero16();
+// The backward kernels share the elementwise work on a summed tile: wave w sums, weighs and packs the registers
+// 4 w .. 4 w + 3 of every lane (a quarter of the tile) and leaves them in LDS as the bytes (w % 2) * 8 .. + 7 of
+// [half w / 2][lane][16 bytes], where every wave then reads the packed operand of its products with two 16-byte reads.
+__device__ __forceinline__ float4 wide_sum_quarter(const char *xch, int wave, int lane) {
+    float4 s = *reinterpret_cast<const float4 *>(xch + wave * 1024 + lane * 16);
 #pragma unroll
-    for (int w = 0; w < 4; ++w)
-#pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4) {
-            const float4 v = *reinterpret_cast<const float4 *>(xch + w * 4096 + r4 * 1024 + lane * 16);
-            X[4 * r4] += v.x;
-            X[4 * r4 + 1] += v.y;
-            X[4 * r4 + 2] += v.z;
-            X[4 * r4 + 3] += v.w;
-        }
-    return X;
+    for (int w = 1; w < 4; ++w) {
+        const float4 v = *reinterpret_cast<const float4 *>(xch + w * 4096 + wave * 1024 + lane * 16);
+        s.x += v.x;
+        s.y += v.y;
+        s.z += v.z;
+        s.w += v.w;
+    }
+    return s;
 }
-
-__device__ __forceinline__ void wide_pack(u32x4 (&pb)[2], const f32x16 &X) {
-#pragma unroll
-    for (int rr = 0; rr < 16; rr += 2) pb[rr >> 3][(rr & 7) >> 1] = pack_bf16(X[rr], X[rr + 1]);
+__device__ __forceinline__ void wide_put_packed(char *pex, int wave, int lane, float a0, float a1, float a2, float a3) {
+    const u32x2 v = {pack_bf16(a0, a1), pack_bf16(a2, a3)};
+    *reinterpret_cast<u32x2 *>(pex + (wave >> 1) * 1024 + lane * 16 + (wave & 1) * 8) = v;
+}
+__device__ __forceinline__ void wide_get_packed(u32x4 (&pb)[2], const char *pex, int lane) {
+    pb[0] = ld_lds16(pex + lane * 16);
+    pb[1] = ld_lds16(pex + 1024 + lane * 16);
 }
 
 // ------------------------------------------------------------------------------------------------------------------
@@ -311,9 +314,11 @@ template <int D>
 __global__ __launch_bounds__(256) void bwd_wide_q_kernel(KParams p, float *ws, int halo) {
     using C = WideCfg<D>;
     constexpr int DB = C::DB, KQ = C::KQ;
-    __shared__ __attribute__((aligned(16))) char lds[4 * C::TILE + 2 * C::XCH];
-    char *tA = lds, *tB = lds + C::TILE, *tK = lds + 2 * C::TILE, *tV = lds + 3 * C::TILE;
-    char *xs = lds + 4 * C::TILE, *xp = xs + C::XCH;
+    // operand tiles A, B; two buffers of K1 / V1 tiles; the exchange areas of the partial tiles; the packed weights
+    __shared__ __attribute__((aligned(16))) char lds[6 * C::TILE + 2 * C::XCH + 2 * 2048];
+    char *tA = lds, *tB = lds + C::TILE;
+    char *xs = lds + 6 * C::TILE, *xp = xs + C::XCH, *pexP = xp + C::XCH, *pexS = pexP + 2048;
+    int buf = 0;
 
     const int N = p.N;
     const int ntile = (N + 31) / 32;
@@ -375,7 +380,9 @@ __global__ __launch_bounds__(256) void bwd_wide_q_kernel(KParams p, float *ws, i
         for (int db = 0; db < DB; ++db) G[db] = T[db] = zero16();
         const bool col_ok = row_ok && i - dlt >= 0;
         for (int t = t_lo; t <= t_hi; ++t) {
-            __syncthreads();
+            // (two tile buffers: a store meets no reader, every wave has passed three barriers since the buffer's last use)
+            char *tK = lds + 2 * C::TILE + buf * 2 * C::TILE, *tV = tK + C::TILE;
+            buf ^= 1;
             wide_store<D>(tK, nk, tid);
             wide_store<D>(tV, nv, tid);
             {
@@ -384,28 +391,36 @@ __global__ __launch_bounds__(256) void bwd_wide_q_kernel(KParams p, float *ws, i
                 wide_pieces<D>(nv, v1g, p.v1.sn, 32 * tn, N, tid);
             }
             __syncthreads();
-            f32x16 X = zero16(), Y = zero16();
+            {
+                f32x16 X = zero16(), Y = zero16();
 #pragma unroll
-            for (int kq = 0; kq < KQ; ++kq) {
-                X = mfma32(sw.row_frag(tK, wave * KQ + kq), sw.row_frag(tA, wave * KQ + kq), X);
-                Y = mfma32(sw.row_frag(tV, wave * KQ + kq), sw.row_frag(tB, wave * KQ + kq), Y);
+                for (int kq = 0; kq < KQ; ++kq) {
+                    X = mfma32(sw.row_frag(tK, wave * KQ + kq), sw.row_frag(tA, wave * KQ + kq), X);
+                    Y = mfma32(sw.row_frag(tV, wave * KQ + kq), sw.row_frag(tB, wave * KQ + kq), Y);
+                }
+                wide_put(xs, wave, lane, X);
+                wide_put(xp, wave, lane, Y);
             }
-            wide_put(xs, wave, lane, X);
-            wide_put(xp, wave, lane, Y);
             __syncthreads();
-            X = wide_sum(xs, lane);
-            Y = wide_sum(xp, lane);
-            const int rel = col_ok ? i - 32 * t - 4 * hf : -(1 << 30);
+            {
+                // this wave's quarter of the tile: key rows j = 32 t + 8 wave + 4 hf + e
+                const float4 x4 = wide_sum_quarter(xs, wave, lane), y4 = wide_sum_quarter(xp, wave, lane);
+                const int rel = col_ok ? i - 32 * t - 4 * hf - 8 * wave : -(1 << 30);
+                const float xe[4] = {x4.x, x4.y, x4.z, x4.w}, ye[4] = {y4.x, y4.y, y4.z, y4.w};
+                float pr[4], ds[4];
 #pragma unroll
-            for (int rr = 0; rr < 16; ++rr) {
-                const bool ok = (unsigned)(rel - (8 * (rr >> 2) + (rr & 3))) < (unsigned)p.w1;
-                const float pr = ok ? fast_exp2(X[rr] - lse2) : 0.f;
-                X[rr] = pr;
-                Y[rr] = pr * (Y[rr] - dl);
+                for (int e = 0; e < 4; ++e) {
+                    const bool ok = (unsigned)(rel - e) < (unsigned)p.w1;
+                    pr[e] = ok ? fast_exp2(xe[e] - lse2) : 0.f;
+                    ds[e] = pr[e] * (ye[e] - dl);
+                }
+                wide_put_packed(pexP, wave, lane, pr[0], pr[1], pr[2], pr[3]);
+                wide_put_packed(pexS, wave, lane, ds[0], ds[1], ds[2], ds[3]);
             }
+            __syncthreads();
             u32x4 pbP[2], pbS[2];
-            wide_pack(pbP, X);
-            wide_pack(pbS, Y);
+            wide_get_packed(pbP, pexP, lane);
+            wide_get_packed(pbS, pexS, lane);
 #pragma unroll
             for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -454,9 +469,9 @@ template <int D>
 __global__ __launch_bounds__(256) void bwd_wide_kv_kernel(KParams p) {
     using C = WideCfg<D>;
     constexpr int DB = C::DB, KQ = C::KQ;
-    __shared__ __attribute__((aligned(16))) char lds[2 * C::TILE + 2 * C::XCH + 2 * 32 * 4];
-    char *tA = lds, *tB = lds + C::TILE, *xs = lds + 2 * C::TILE, *xp = xs + C::XCH;
-    float *lse_s = reinterpret_cast<float *>(xp + C::XCH), *del_s = lse_s + 32;
+    __shared__ __attribute__((aligned(16))) char lds[2 * C::TILE + 2 * C::XCH + 2 * 2048 + 2 * 32 * 4];
+    char *tA = lds, *tB = lds + C::TILE, *xs = lds + 2 * C::TILE, *xp = xs + C::XCH, *pexP = xp + C::XCH, *pexS = pexP + 2048;
+    float *lse_s = reinterpret_cast<float *>(pexS + 2048), *del_s = lse_s + 32;
 
     const int N = p.N;
     const int ntile = (N + 31) / 32;
@@ -520,35 +535,39 @@ __global__ __launch_bounds__(256) void bwd_wide_kv_kernel(KParams p) {
                 wide_pieces<D>(nyv, v2g, p.v2.sn, i0 - dlt - 1, N, tid);
                 __syncthreads();
                 // S[i][j], dP[i][j]: register rr of this lane is query row i0 + 8 (rr / 4) + 4 hf + rr % 4, the lane's column is key row j
-                f32x16 X = zero16(), Y = zero16();
+                {
+                    f32x16 X = zero16(), Y = zero16();
 #pragma unroll
-                for (int kq = 0; kq < KQ; ++kq) {
-                    X = mfma32(sw.row_frag(tA, wave * KQ + kq), kfr[kq], X);
-                    Y = mfma32(sw.row_frag(tB, wave * KQ + kq), vfr[kq], Y);
+                    for (int kq = 0; kq < KQ; ++kq) {
+                        X = mfma32(sw.row_frag(tA, wave * KQ + kq), kfr[kq], X);
+                        Y = mfma32(sw.row_frag(tB, wave * KQ + kq), vfr[kq], Y);
+                    }
+                    wide_put(xs, wave, lane, X);
+                    wide_put(xp, wave, lane, Y);
                 }
-                wide_put(xs, wave, lane, X);
-                wide_put(xp, wave, lane, Y);
                 __syncthreads();
-                X = wide_sum(xs, lane);
-                Y = wide_sum(xp, lane);
-#pragma unroll
-                for (int q4 = 0; q4 < 4; ++q4) {
-                    const float4 l4 = *reinterpret_cast<const float4 *>(lse_s + 8 * q4 + 4 * hf);
-                    const float4 d4 = *reinterpret_cast<const float4 *>(del_s + 8 * q4 + 4 * hf);
-                    const float ls[4] = {l4.x, l4.y, l4.z, l4.w}, ds[4] = {d4.x, d4.y, d4.z, d4.w};
+                {
+                    // this wave's quarter of the tile: query rows i0 + 8 wave + 4 hf + e
+                    const float4 x4 = wide_sum_quarter(xs, wave, lane), y4 = wide_sum_quarter(xp, wave, lane);
+                    const float4 l4 = *reinterpret_cast<const float4 *>(lse_s + 8 * wave + 4 * hf);
+                    const float4 d4 = *reinterpret_cast<const float4 *>(del_s + 8 * wave + 4 * hf);
+                    const float xe[4] = {x4.x, x4.y, x4.z, x4.w}, ye[4] = {y4.x, y4.y, y4.z, y4.w};
+                    const float le[4] = {l4.x, l4.y, l4.z, l4.w}, de[4] = {d4.x, d4.y, d4.z, d4.w};
+                    float pr[4], ds[4];
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        const int rr = 4 * q4 + e;
-                        const int ii = i0 + 8 * q4 + 4 * hf + e;
+                        const int ii = i0 + 8 * wave + 4 * hf + e;
                         const bool ok = ii < N && ii - dlt >= 0 && (unsigned)(ii - j) < (unsigned)p.w1;
-                        const float pr = ok ? fast_exp2(X[rr] - ls[e]) : 0.f;
-                        X[rr] = pr;
-                        Y[rr] = pr * (Y[rr] - ds[e]);
+                        pr[e] = ok ? fast_exp2(xe[e] - le[e]) : 0.f;
+                        ds[e] = pr[e] * (ye[e] - de[e]);
                     }
+                    wide_put_packed(pexP, wave, lane, pr[0], pr[1], pr[2], pr[3]);
+                    wide_put_packed(pexS, wave, lane, ds[0], ds[1], ds[2], ds[3]);
                 }
+                __syncthreads();
                 u32x4 pbP[2], pbS[2];
-                wide_pack(pbP, X);
-                wide_pack(pbS, Y);
+                wide_get_packed(pbP, pexP, lane);
+                wide_get_packed(pbS, pexS, lane);
 #pragma unroll
                 for (int db = 0; db < DB; ++db)
 #pragma unroll
