@@ -266,6 +266,38 @@ def vendor_gemm_rates(n=8192, iters=10):
     return res
 
 
+def vendor_attention_rates(B=4, H=8, N=8192, D=128, iters=5):
+    """A third calibration point: torch's scaled_dot_product_attention (the vendor's fused attention kernels) on random
+    bf16 inputs at config 3's batch, heads, length and head dimension, causal, forward and forward + backward.
+    Flop: 4 N^2 D B H / 2 forward, 2.5 times that for the backward."""
+    import torch
+    import torch.nn.functional as F
+    dev = torch.device('cuda:0')
+    g = torch.Generator(device='cpu').manual_seed(5)
+    q, k, v = ((torch.randn(B, H, N, D, generator=g) * D ** -0.25).bfloat16().to(dev).requires_grad_(True) for _ in range(3))
+    do = torch.randn(B, H, N, D, generator=g).bfloat16().to(dev)
+    fwd_flop = 4 * N * N * D * B * H / 2
+
+    def timed(fn):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(iters):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) / iters
+
+    with torch.no_grad():
+        t_f = timed(lambda: F.scaled_dot_product_attention(q, k, v, is_causal=True))
+    t_fb = timed(lambda: torch.autograd.grad(F.scaled_dot_product_attention(q, k, v, is_causal=True), (q, k, v), do))
+    res = {'fwd': {'ms': round(t_f * 1e3, 3), 'tflops': round(fwd_flop / t_f / 1e12, 1)},
+           'fwd_bwd': {'ms': round(t_fb * 1e3, 3), 'tflops': round(3.5 * fwd_flop / t_fb / 1e12, 1)}}
+    for r in res.values():
+        r['frac_of_nominal_peak'] = round(r['tflops'] / PEAK_BF16_TFLOPS, 4)
+    return res
+
+
 def time_raw_workload(name, steps=5, warmup=2):
     """forward + backward of the raw kernel path at workload `name` through the autograd Function: ms per step,
     TFLOP/s on the 18*D*B*H*P count and the fraction of the bf16 MFMA peak."""
@@ -426,7 +458,8 @@ def main():
         print(json.dumps(time_module_cfg2()))
         return
     if args.only == 'mfma_mix':
-        print(json.dumps({'instruction_mix_loop': mfma_mix_rates(), 'torch_matmul_bf16_8192': vendor_gemm_rates()}))
+        print(json.dumps({'instruction_mix_loop': mfma_mix_rates(), 'torch_matmul_bf16_8192': vendor_gemm_rates(),
+                          'torch_sdpa_causal_b4_h8_n8192_d128': vendor_attention_rates()}))
         return
     if args.only == 'copy':
         # plain device copy of known size: calibrates the FETCH_SIZE / WRITE_SIZE counters
