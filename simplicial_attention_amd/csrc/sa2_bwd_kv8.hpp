@@ -582,8 +582,6 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
             dP[4 * a4 + 2] = d4.z;
             dP[4 * a4 + 3] = d4.w;
         }
-        mfma_stream(NChain{}, [&](auto kk) { return swz_lane.row_frag(buf + L::BS, kk); },
-                    [&](auto kk, const u32x4 &fr) { dP = mfma32(fr, v1f[kk], dP); });
         const bool full = (jw + 31 <= 32 * it) && (jw + p.w1 > 32 * it + 31);
         if (__builtin_expect(!full, 0)) {
             int base = 32 * it + 4 * hf - j;         // i - j for register 0
@@ -594,19 +592,32 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
                 X[rr] = ok ? X[rr] : -INFINITY;
             }
         }
+        // The VALU work rides behind MFMAs that do not depend on it: the exponentials of S behind the dP chain, dS = P dP
+        // behind the dV1 products (which take P), and the dK1 products last.
+        constexpr int NPER = 16 / KS;              // logits per MFMA of a chain (KS = 2 DT MFMAs per chain and per product)
         u32x4 pb[2];                 // dS
         u32x4 pv[2];                 // P
+        mfma_stream2(NChain{}, [&](auto kk) { return swz_lane.row_frag(buf + L::BS, kk); },
+                     [&](auto kk, const u32x4 &fr) { dP = mfma32(fr, v1f[kk], dP); },
+                     [&](auto x_) {
+                         constexpr int x = decltype(x_)::value;
 #pragma unroll
-        for (int rr = 0; rr < 16; rr += 2) {
-            const float p0 = fast_exp2(X[rr]);
-            const float p1 = fast_exp2(X[rr + 1]);
-            pv[rr >> 3][(rr & 7) >> 1] = pack_bf16(p0, p1);
-            pb[rr >> 3][(rr & 7) >> 1] = pack_bf16(p0 * dP[rr], p1 * dP[rr + 1]);
-        }
+                         for (int rr = NPER * x; rr < NPER * (x + 1); rr += 2) {
+                             X[rr] = fast_exp2(X[rr]);
+                             X[rr + 1] = fast_exp2(X[rr + 1]);
+                             pv[rr >> 3][(rr & 7) >> 1] = pack_bf16(X[rr], X[rr + 1]);
+                         }
+                     });
+        mfma_stream2(NProd{}, [&](auto x) { return swz_lane.tr_frag(buf + L::BS, x / DT, x % DT); },
+                     [&](auto x, const u32x4 &fr) { acc2[x % DT] = mfma32(fr, pv[x / DT], acc2[x % DT]); },
+                     [&](auto x_) {
+                         constexpr int x = decltype(x_)::value;
+#pragma unroll
+                         for (int rr = NPER * x; rr < NPER * (x + 1); rr += 2)
+                             pb[rr >> 3][(rr & 7) >> 1] = pack_bf16(X[rr] * dP[rr], X[rr + 1] * dP[rr + 1]);
+                     });
         mfma_stream(NProd{}, [&](auto x) { return swz_lane.tr_frag(buf + L::AS, x / DT, x % DT); },
                     [&](auto x, const u32x4 &fr) { acc[x % DT] = mfma32(fr, pb[x / DT], acc[x % DT]); });
-        mfma_stream(NProd{}, [&](auto x) { return swz_lane.tr_frag(buf + L::BS, x / DT, x % DT); },
-                    [&](auto x, const u32x4 &fr) { acc2[x % DT] = mfma32(fr, pv[x / DT], acc2[x % DT]); });
     }
 
     // ---- add the two groups of every slab and store
