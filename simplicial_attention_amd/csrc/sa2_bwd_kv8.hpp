@@ -93,7 +93,10 @@ __global__ __launch_bounds__(512) void bwd_kv8_kernel(KParams p) {
 
     const int tid = threadIdx.x;
     const int wave = wave_index(), lane = tid & 63;
-    const int slab = wave & 3, pg = wave >> 2;
+    // The two waves of a slab sit on different SIMDs (wave w runs on SIMD w % 4): in the query tiles at both ends of a
+    // workgroup's walk, which only one or two of its slabs reach, the active waves then have a SIMD each instead of
+    // sharing one while others idle.  In the other tiles every SIMD still holds one wave of each group.
+    const int pg = wave >> 2, slab = ((wave & 3) + 2 * pg) & 3;
     const int c = lane & 31, hf = lane >> 5;
     const int j0 = tile * 128;
     const int jw = j0 + 32 * slab;
